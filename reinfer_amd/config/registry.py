@@ -3,7 +3,7 @@
 A configuration class has ``from_dict(config_json) -> cfg``, ``cfg.to_dict()``
 and ``cfg.to_spec() -> ModelSpec``. The name is ``architectures[0]`` of
 config.json, else ``model_type`` (the reference selects the same way,
-crates/arch/src/llama.rs:305-317).
+crates/arch/src/llama.rs:305-317), else the string under ``architecture``.
 """
 from __future__ import annotations
 
@@ -32,6 +32,9 @@ def architecture_name(cfg: Mapping[str, Any]) -> str:
     mt = cfg.get("model_type", None)
     if isinstance(mt, str):
         return mt
+    one = cfg.get("architecture", None)          # a configuration that names its one architecture in a string
+    if isinstance(one, str):
+        return one
     raise ConfigError("architectures", "required key is missing")
 
 

@@ -137,6 +137,60 @@ class FeedForwardSpec:
 
 
 @dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Sizes of an attention whose keys and values are linear maps of one cached latent vector a token
+    (``MixerSpec.params`` of the "latent_attention" mixer; heads, scale, window and rotation are the
+    ``MixerSpec``'s own fields): a query head is ``head_dim`` unrotated and ``rot_width`` rotated entries, the
+    latent ``rank`` wide, a value head ``value_dim``; ``gated``: the concatenated heads are multiplied by the
+    sigmoid of a projection of the mixer's input before the output projection."""
+    rank: int
+    rot_width: int
+    value_dim: int
+    norm_eps: float
+    gated: bool = True
+
+
+@dataclass(frozen=True)
+class MoESpec:
+    """Routing of a mixture-of-experts feed-forward (``FeedForwardSpec.params``; ``intermediate`` is one
+    expert's width): ``experts`` of which each token uses ``top``; ``activation`` of an expert ("relu2": the
+    square of relu, no gate); ``weights``: "softmax_chosen" = softmax over the chosen logits alone."""
+    experts: int
+    top: int
+    activation: str = "relu2"
+    weights: str = "softmax_chosen"
+
+
+@dataclass(frozen=True)
+class InputSpec:
+    """Something added to the token embedding before the first layer, beyond positions: ``kind`` picks the
+    part (registry "input"), ``params`` is the part's own typed record, ``prefix`` goes before its tensor
+    names."""
+    kind: str
+    params: Any = None
+    prefix: str = ""
+
+
+@dataclass(frozen=True)
+class PairHashSpec:
+    """A table of ``buckets`` + 1 rows looked up by a hash of (previous token, token):
+    row = (previous * mul_prev + token * mul_cur) mod buckets; a request's first token takes the last row."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    table_name: str = "bigram"
+
+
+@dataclass(frozen=True)
+class StreamAdd:
+    """What is added to the residual stream right before a run-order entry: the embedding output once more
+    (``embedding``), and row ``row`` of the [rows, width] tensor ``vector`` (None: no vector)."""
+    embedding: bool = False
+    vector: Optional[str] = None
+    row: int = 0
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: how norm, mixer and feed-forward are arranged, and its parts.
 
@@ -170,6 +224,7 @@ class RunEntry:
     """
     block: int
     cache_from: Optional[int] = None
+    before: Optional[StreamAdd] = None      # added to the stream right before this entry runs
 
 
 @dataclass(frozen=True)
@@ -191,11 +246,22 @@ class ModelSpec:
     # architectures whose mixers do not rotate; None: positions enter in the mixers only
     input_position: Optional[PositionSpec] = None
     input_position_prefix: str = "model."
+    # further parts that add to the embedding (a hashed token-pair table, ...), in order
+    inputs: Tuple[InputSpec, ...] = ()
+    # [rows, width] tensors whose rows run-order entries add to the stream (``RunEntry.before``): (name, rows)
+    stream_vectors: Tuple[Tuple[str, int], ...] = ()
+    # logits <- cap * tanh(logits / cap) when cap > 0
+    logit_softcap: float = 0.0
 
     def __post_init__(self):
         for i, e in enumerate(self.run_order):
             if not 0 <= e.block < len(self.blocks):
                 raise ConfigError("run_order", f"entry {i} names block {e.block} of {len(self.blocks)}")
+            if e.before is not None and e.before.vector is not None:
+                rows = dict(self.stream_vectors).get(e.before.vector)
+                if rows is None or not 0 <= e.before.row < rows:
+                    raise ConfigError("run_order", f"entry {i} adds row {e.before.row} of {e.before.vector!r}, "
+                                                   "which the model does not declare")
             if e.cache_from is not None:
                 if not 0 <= e.cache_from < i:
                     raise ConfigError("run_order", f"entry {i} reads the cache of entry {e.cache_from}, "

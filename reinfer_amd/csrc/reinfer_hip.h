@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 17
+#define RA_ABI_VERSION 18
 
 #ifdef __cplusplus
 extern "C" {
@@ -164,6 +164,42 @@ int ra_filter_logits(float* logits, int n_rows, int vocab, int row_stride, const
 // device memory that is never written in practice.
 int ra_stream_read(const void* src, long bytes, void* sink, hipStream_t stream);
 int ra_mfma_loop(int shape, int iters, int waves_per_cu, void* sink, double* flops, hipStream_t stream);
+
+// ---- around the residual stream (stream.hip) ----
+// resid[t, :] += table[row(t), :] with row(t) = (prev * mul_prev + id * mul_cur) mod buckets, row `buckets` for a
+// request's first token (position 0). The token before a portion's first comes from last_token[state slot of the
+// request], which is then set to the portion's last token; state slot -1 reads and writes nothing.
+int ra_pair_hash_add(float* resid, const void* table, int table_dtype, const int* ids, const int* positions,
+                     const int* seq_of_token, const int* cu_tokens, const int* state_slots, int* last_token,
+                     int buckets, long long mul_prev, long long mul_cur, int n_tokens, int hidden,
+                     hipStream_t stream);
+// resid[t, :] += delta[t, :] + other[t, :] + vec[:]; every addend may be null
+int ra_stream_add(float* resid, const void* delta, int delta_dtype, const float* other, const void* vec,
+                  int vec_dtype, int n_tokens, int hidden, hipStream_t stream);
+// logits <- cap * tanh(logits / cap) in place
+int ra_tanh_cap(float* logits, int n_rows, int vocab, int row_stride, float cap, hipStream_t stream);
+
+// ---- attention over a shared latent (latent.hip) ----
+// proj rows hold H query heads ([D unrotated | R rotated] each) from column q_off and [c_raw (rank) | kr (R)] from
+// column dkv_off. Writes the cache row [rms(c_raw) * c_weight | rot(kr) | 0...] of Dp (a multiple of 16) elements in
+// the K and V tile layouts of one KV head at slots[t] (-1: nothing), and q_lat[t, h, rank:Dp] = [rot(q_h's rotated
+// part) | 0...]. Rotation: the first rot_dims of an R-wide part, half-split pairs, angle pos * inv_freq[i].
+int ra_latent_prep(const void* proj, int act_dtype, int ld, int q_off, int dkv_off, const void* c_weight,
+                   int weight_dtype, float eps, const int* positions, const float* inv_freq, int rot_dims, int R,
+                   int rank, int H, int D, void* q_lat, int Dp, const int* slots, void* kcache, void* vcache,
+                   int block_size, int n_tokens, hipStream_t stream);
+// out[t, h * o_head + n] = sum_k x[t, h * x_head + k] * W[h, k, n] (* sigmoid(gate[t, h * N + n]) if gate)
+int ra_head_linear(const void* x, int ldx, int x_head, const void* W, void* out, int ldo, int o_head,
+                   const void* gate, int ldg, int act_dtype, int n_tokens, int H, int N, int K, hipStream_t stream);
+
+// ---- mixture of experts (moe.hip) ----
+// float router logits of x [n_tokens, width] against router [experts, width] (float), the `top` (<= 64) largest
+// in falling order into ids [n_tokens, top], their softmax over the chosen alone into weights [n_tokens, top]
+int ra_moe_route(const void* x, int act_dtype, int ldx, const float* router, int experts, int width, int top,
+                 int* ids, float* weights, int n_tokens, hipStream_t stream);
+// act[t, e * ff + j] = weight(t, e) * relu(up[t, e * ff + j])^2 for chosen experts, 0 for the others
+int ra_moe_relu2_scale(const void* up, void* act, int act_dtype, const int* ids, const float* weights, int top,
+                       int experts, int ff, int n_tokens, hipStream_t stream);
 
 #ifdef __cplusplus
 }

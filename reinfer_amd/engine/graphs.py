@@ -116,7 +116,7 @@ class _CapturedStep:
 
     def _body(self) -> None:
         r = self.runner
-        self.logits = r.model.forward(self.batch, r.caches)
+        self.logits = r.model.forward(self.batch, r.caches, None, r.input_states)
         kernels.current().sample(self.logits, self.temps, self.seeds, self.sample_pos, self.tokens)
 
     def _capture(self, pool) -> None:

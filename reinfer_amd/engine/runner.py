@@ -102,6 +102,12 @@ class ModelRunner:
             else:
                 self.caches.append(None)
 
+        # per-request state of the parts at the embedding (one tensor [max_seqs, *shape] each, indexed by the
+        # step's state slots like a layer's state)
+        self.input_states: List[Optional[torch.Tensor]] = [
+            torch.zeros((max_seqs, *need.shape), dtype=need.dtype, device=device) if need is not None else None
+            for need in self.model.input_needs()]
+
         # decode steps replay captured graphs when every part says it can be captured
         # (a block arrangement says so itself with ``graph_safe``, or it is asked of its ``mixer`` and ``ffn``)
         def block_safe(b) -> bool:
@@ -110,7 +116,8 @@ class ModelRunner:
             return bool(getattr(getattr(b, "mixer", None), "graph_safe", False)
                         and getattr(getattr(b, "ffn", None), "graph_safe", False))
         safe = all(block_safe(b) for b in self.model.blocks) and \
-            (self.model.input_position is None or bool(getattr(self.model.input_position, "graph_safe", False)))
+            (self.model.input_position is None or bool(getattr(self.model.input_position, "graph_safe", False))) \
+            and all(bool(getattr(p, "graph_safe", False)) for p in self.model.inputs)
         if use_graphs is None:
             use_graphs = True
         self.graphs = None
@@ -283,6 +290,6 @@ class ModelRunner:
         with torch.no_grad():
             if batch.num_logit_rows == 0:
                 # still run the layers: the step's keys and values must be stored
-                self.model.forward_layers(batch, self.caches, observer)
+                self.model.forward_layers(batch, self.caches, observer, self.input_states)
                 return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-            return self.model.forward(batch, self.caches, observer)
+            return self.model.forward(batch, self.caches, observer, self.input_states)

@@ -8,14 +8,14 @@ from __future__ import annotations
 
 import ctypes
 import threading
-from ctypes import c_char_p, c_float, c_int, c_long, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_longlong, c_void_p
 from typing import Optional
 
 import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 
 class KernelLibraryError(RuntimeError):
@@ -47,6 +47,13 @@ _SIGNATURES = {
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],
     "ra_sample_static": [P, I, I, I, P, P, P, P, P],
     "ra_filter_logits": [P, I, I, I, P, P, P],
+    "ra_pair_hash_add": [P, P, I, P, P, P, P, P, P, I, c_longlong, c_longlong, I, I, P],
+    "ra_stream_add": [P, P, I, P, P, I, I, I, P],
+    "ra_tanh_cap": [P, I, I, I, F, P],
+    "ra_latent_prep": [P, I, I, I, I, P, I, F, P, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
+    "ra_head_linear": [P, I, I, P, P, I, I, P, I, I, I, I, I, I, P],
+    "ra_moe_route": [P, I, I, P, I, I, I, P, P, I, P],
+    "ra_moe_relu2_scale": [P, P, I, P, P, I, I, I, I, P],
     "ra_stream_read": [P, c_long, P, P],
     "ra_mfma_loop": [I, I, I, P, P, P],
 }

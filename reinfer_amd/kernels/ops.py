@@ -840,6 +840,148 @@ class HipKernels:
         self.linear(x, weight, gu)
         self.silu_mul(gu, out, self.GATE_GROUP)
 
+    # ------------------------------------------------- around the stream
+    def pair_hash_add(self, resid: torch.Tensor, table: torch.Tensor, batch, last_token: torch.Tensor,
+                      buckets: int, mul_prev: int, mul_cur: int) -> None:
+        """resid[t] += table[(prev * mul_prev + id * mul_cur) mod buckets], or the table's last row (number
+        ``buckets``) for a request's first token. The token before a portion's first is read from
+        ``last_token[state slot]`` (int32, one word a request slot), which then takes the portion's last token."""
+        _dev(resid, table, last_token)
+        T, h = resid.shape
+        if T != batch.num_tokens or resid.dtype != torch.float32 or not resid.is_contiguous():
+            raise TypeError("pair_hash_add: the residual stream is contiguous float32, one row a token of the step")
+        if table.shape != (buckets + 1, h) or not table.is_contiguous():
+            raise ValueError(f"pair_hash_add: table {tuple(table.shape)}, expected [{buckets + 1}, {h}]")
+        _int32(last_token, "pair_hash_add state")
+        slots_needed = int(last_token.numel())
+        if slots_needed <= 0:
+            raise ValueError("pair_hash_add: no state words")
+        _int32(batch.token_ids, "token ids", T)
+        _int32(batch.positions, "positions", T)
+        _int32(batch.seq_of_token, "request of each token", T)
+        _int32(batch.cu_tokens, "first token of each request", batch.num_seqs + 1)
+        _int32(batch.state_slots, "state slots", batch.num_seqs)
+        library.call("ra_pair_hash_add", resid.data_ptr(), table.data_ptr(), _tag(table, "pair table"),
+                     batch.token_ids.data_ptr(), batch.positions.data_ptr(), batch.seq_of_token.data_ptr(),
+                     batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), last_token.data_ptr(), int(buckets),
+                     int(mul_prev), int(mul_cur), T, h, _stream())
+
+    def stream_add(self, resid: torch.Tensor, delta: Optional[torch.Tensor] = None,
+                   other: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None) -> None:
+        """resid += delta + other + vec: ``delta`` [T, width] in either dtype, ``other`` [T, width] float32,
+        ``vec`` [width] in either dtype; each may be None."""
+        _dev(resid, delta, other, vec)
+        T, h = resid.shape
+        if resid.dtype != torch.float32 or not resid.is_contiguous():
+            raise TypeError("stream_add: the residual stream is contiguous float32")
+        if delta is not None and (delta.shape != resid.shape or not delta.is_contiguous()):
+            raise ValueError("stream_add: delta must match the residual's shape")
+        if other is not None and (other.shape != resid.shape or other.dtype != torch.float32 or not other.is_contiguous()):
+            raise ValueError("stream_add: the second addend is a float32 matrix of the residual's shape")
+        if vec is not None and (vec.shape != (h,) or not vec.is_contiguous()):
+            raise ValueError(f"stream_add: vector {tuple(vec.shape)}, expected [{h}]")
+        if delta is None and other is None and vec is None:
+            return
+        library.call("ra_stream_add", resid.data_ptr(), _ptr(delta), _tag(delta, "stream_add delta") if delta is not None else 0,
+                     _ptr(other), _ptr(vec), _tag(vec, "stream_add vector") if vec is not None else 0, T, h, _stream())
+
+    def tanh_cap(self, logits: torch.Tensor, cap: float) -> None:
+        """logits <- cap * tanh(logits / cap), in place."""
+        _dev(logits)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+            raise TypeError("tanh_cap: logits are float32 rows")
+        if logits.shape[0] == 0:
+            return
+        library.call("ra_tanh_cap", logits.data_ptr(), logits.shape[0], logits.shape[1], logits.stride(0),
+                     float(cap), _stream())
+
+    # ------------------------------------------------------ latent attention
+    def latent_prep(self, proj: torch.Tensor, q_off: int, dkv_off: int, c_weight: torch.Tensor, eps: float,
+                    positions: torch.Tensor, inv_freq: torch.Tensor, rot_dims: int, rot_width: int, rank: int,
+                    num_heads: int, head_dim: int, q_lat: torch.Tensor, slots: torch.Tensor,
+                    kcache: torch.Tensor, vcache: torch.Tensor) -> None:
+        """Norm of the latent, rotation of the shared key part and of the queries' rotated parts, cache write.
+
+        ``proj`` [T, *] holds the query heads ([head_dim | rot_width] each) from column ``q_off`` and
+        [latent (rank) | key part (rot_width)] from ``dkv_off``. The cache row of a token,
+        [rms(latent) * c_weight | rotated key part | zeros], goes to ``kcache`` / ``vcache`` (one KV head of
+        size Dp = q_lat.shape[2]) at ``slots``; ``q_lat`` [T, heads, Dp] gets its columns from ``rank`` on."""
+        _dev(proj, c_weight, positions, inv_freq, q_lat, slots, kcache, vcache)
+        T = proj.shape[0]
+        if proj.dim() != 2 or proj.stride(1) != 1:
+            raise ValueError("latent_prep: projection rows must be contiguous")
+        if q_lat.dim() != 3 or q_lat.shape[:2] != (T, num_heads) or not q_lat.is_contiguous() or q_lat.dtype != proj.dtype:
+            raise ValueError(f"latent_prep: q_lat {tuple(q_lat.shape)}, expected [{T}, {num_heads}, Dp] in the activations' dtype")
+        Dp = q_lat.shape[2]
+        self._check_cache("latent_prep", kcache, vcache, 1, Dp)
+        if kcache.dtype != proj.dtype or vcache.dtype != proj.dtype:
+            raise TypeError("latent_prep: the cache has the activations' dtype")
+        if c_weight.shape != (rank,) or not c_weight.is_contiguous():
+            raise ValueError(f"latent_prep: norm weight {tuple(c_weight.shape)}, expected [{rank}]")
+        _int32(positions, "positions", T)
+        _int32(slots, "cache slots", T)
+        if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(1, rot_dims // 2):
+            raise ValueError("latent_prep: inv_freq is float32 with rot_dims/2 entries")
+        library.call("ra_latent_prep", proj.data_ptr(), _tag(proj, "latent_prep"), proj.stride(0), int(q_off),
+                     int(dkv_off), c_weight.data_ptr(), _tag(c_weight, "latent norm weight"), float(eps),
+                     positions.data_ptr(), inv_freq.data_ptr(), int(rot_dims), int(rot_width), int(rank),
+                     int(num_heads), int(head_dim), q_lat.data_ptr(), Dp, slots.data_ptr(), kcache.data_ptr(),
+                     vcache.data_ptr(), kcache.shape[2] * 16, T, _stream())
+
+    def head_linear(self, x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, o_head: int,
+                    gate: Optional[torch.Tensor] = None) -> None:
+        """Products head by head: out[t, h * o_head + n] = sum_k x[t, h * x_head + k] * weight[h, k, n], times
+        sigmoid(gate[t, h * N + n]) where a gate is given. ``x``, ``out`` and ``gate`` are 2-D with unit
+        column stride (they may be column ranges of wider buffers); ``weight`` is [heads, K, N] contiguous."""
+        _dev(x, weight, out, gate)
+        H, K, N = weight.shape
+        T = x.shape[0]
+        if not weight.is_contiguous() or x.dtype != weight.dtype or out.dtype != weight.dtype:
+            raise ValueError("head_linear: weight [heads, K, N] contiguous, all in one dtype")
+        for t, what in ((x, "x"), (out, "out"), (gate, "gate")):
+            if t is not None and (t.dim() != 2 or t.shape[0] != T or t.stride(1) != 1 or t.dtype != weight.dtype):
+                raise ValueError(f"head_linear: {what} must be [T, *] rows of the weight's dtype with unit column stride")
+        if x.shape[1] < (H - 1) * x_head + K or out.shape[1] < (H - 1) * o_head + N or o_head < N:
+            raise ValueError(f"head_linear: x {tuple(x.shape)} / out {tuple(out.shape)} do not hold {H} heads of {K} / {N}")
+        if gate is not None and gate.shape[1] < H * N:
+            raise ValueError(f"head_linear: gate {tuple(gate.shape)}, expected [T, {H * N}]")
+        library.call("ra_head_linear", x.data_ptr(), x.stride(0), int(x_head), weight.data_ptr(), out.data_ptr(),
+                     out.stride(0), int(o_head), _ptr(gate), gate.stride(0) if gate is not None else 0,
+                     _tag(x, "head_linear"), T, H, N, K, _stream())
+
+    # ---------------------------------------------------- mixture of experts
+    def moe_route(self, x: torch.Tensor, router: torch.Tensor, top: int, ids: torch.Tensor,
+                  weights: torch.Tensor) -> None:
+        """Float router logits x . router^T, the ``top`` largest a token in falling order into ``ids`` [T, top]
+        (int32) and the softmax over those alone into ``weights`` [T, top] (float32)."""
+        _dev(x, router, ids, weights)
+        T, width = x.shape
+        E = router.shape[0]
+        if router.shape != (E, width) or router.dtype != torch.float32 or not router.is_contiguous():
+            raise ValueError(f"moe_route: router {tuple(router.shape)} {router.dtype}, expected float32 [experts, {width}]")
+        if x.stride(1) != 1:
+            raise ValueError("moe_route: rows must be contiguous")
+        if ids.shape != (T, top) or ids.dtype != torch.int32 or not ids.is_contiguous() \
+                or weights.shape != (T, top) or weights.dtype != torch.float32 or not weights.is_contiguous():
+            raise ValueError(f"moe_route: ids int32 and weights float32, both [{T}, {top}]")
+        library.call("ra_moe_route", x.data_ptr(), _tag(x, "moe_route"), x.stride(0), router.data_ptr(), E, width,
+                     int(top), ids.data_ptr(), weights.data_ptr(), T, _stream())
+
+    def moe_relu2_scale(self, up: torch.Tensor, act: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+                        experts: int, ff: int) -> None:
+        """act[t, e * ff + j] = weight(t, e) * relu(up[t, e * ff + j])^2 for the chosen experts, 0 for the rest."""
+        _dev(up, act, ids, weights)
+        T = up.shape[0]
+        top = ids.shape[1]
+        if up.shape != (T, experts * ff) or act.shape != up.shape or act.dtype != up.dtype \
+                or not up.is_contiguous() or not act.is_contiguous():
+            raise ValueError(f"moe_relu2_scale: up {tuple(up.shape)} / act {tuple(act.shape)}, expected [T, {experts * ff}]")
+        if ids.shape != (T, top) or ids.dtype != torch.int32 or weights.shape != (T, top) \
+                or weights.dtype != torch.float32 or not ids.is_contiguous() or not weights.is_contiguous():
+            raise ValueError("moe_relu2_scale: ids int32 and weights float32, both [T, top]")
+        library.call("ra_moe_relu2_scale", up.data_ptr(), act.data_ptr(), _tag(up, "moe_relu2_scale"), ids.data_ptr(),
+                     weights.data_ptr(), top, int(experts), int(ff), T, _stream())
+
     # -------------------------------------------------------------- sampling
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, seeds: torch.Tensor,
                positions: torch.Tensor, tokens: torch.Tensor) -> None:

@@ -21,6 +21,10 @@ def declare_params(spec: ModelSpec) -> List[ParamDecl]:
         part = lookup("position", spec.input_position.kind)
         if hasattr(part, "declare_input_params"):
             out += part.declare_input_params(spec.input_position, spec.input_position_prefix)
+    for inp in spec.inputs:
+        out += lookup("input", inp.kind).declare_params(inp, spec.hidden)
+    for name, rows in spec.stream_vectors:
+        out.append(ParamDecl(name, (rows, spec.hidden)))
     for b in spec.blocks:
         out += lookup("block", b.kind).declare_params(b)
     out += lookup("norm", spec.final_norm.kind).declare_params(spec.final_norm, spec.final_norm_name)
@@ -51,6 +55,12 @@ class DecoderModel:
                                  "it has no add_to_stream(resid, batch)")
             self.input_position = part(spec.input_position, device, weights=weights,
                                        prefix=spec.input_position_prefix, dtype=dtype)
+        # further parts that add to the embedding; one that keeps per-request state says so (``state_need()``)
+        # and is handed that state by whoever runs the model (``input_states``, in the order of ``inputs``)
+        self.inputs = [lookup("input", inp.kind)(inp, weights, spec.hidden, dtype, device) for inp in spec.inputs]
+        # rows that run-order entries add to the stream, and whether any of them adds the embedding again
+        self.stream_vectors = {name: weights[name] for name, _ in spec.stream_vectors}
+        self.keeps_embedding = any(e.before is not None and e.before.embedding for e in spec.run_order)
         self.blocks = [lookup("block", b.kind)(b, weights, dtype, device) for b in spec.blocks]
         self.final_norm = lookup("norm", spec.final_norm.kind)(spec.final_norm, weights,
                                                                spec.final_norm_name, dtype, device)
@@ -80,6 +90,8 @@ class DecoderModel:
                 seen.add(id(p))
                 out.append(p)
         add(self.input_position)
+        for p in self.inputs:
+            add(p)
         for b in self.blocks:
             add(b)
             for p in (b.parts() if hasattr(b, "parts") else (getattr(b, "mixer", None), getattr(b, "ffn", None))):
@@ -97,7 +109,11 @@ class DecoderModel:
             if hook is not None:
                 hook(batch, num_rows, ctx_cap)
 
-    def forward_layers(self, batch, caches: Sequence[Optional[LayerCache]], observer=None):
+    def input_needs(self) -> List[Optional[StateNeed]]:
+        """Per-request state that each input part keeps (None: none), in the order of ``inputs``."""
+        return [p.state_need() if hasattr(p, "state_need") else None for p in self.inputs]
+
+    def forward_layers(self, batch, caches: Sequence[Optional[LayerCache]], observer=None, input_states=None):
         """Embedding and all blocks: (residual stream, last addend not yet added).
 
         ``observer(i, hidden)``, if given, is called with the float32 hidden state [T, hidden] behind
@@ -108,12 +124,22 @@ class DecoderModel:
         ops.embed(self.embed, batch.token_ids, resid)
         if self.input_position is not None:
             self.input_position.add_to_stream(resid, batch)
+        for k, part in enumerate(self.inputs):
+            part.add_to_stream(resid, batch, input_states[k] if input_states is not None else None)
         if observer is not None:
             observer(0, resid.clone())
+        embedded = resid.clone() if self.keeps_embedding else None
         delta = None
         n = len(self.run_order)
         for i, e in enumerate(self.run_order):
             block = self.blocks[e.block]
+            if e.before is not None:
+                # what the run order adds ahead of this entry, together with the last block's pending addend
+                if delta is not None and not isinstance(delta, torch.Tensor):
+                    delta = None
+                ops.stream_add(resid, delta, embedded if e.before.embedding else None,
+                               self.stream_vectors[e.before.vector][e.before.row] if e.before.vector else None)
+                delta = None
             # the block that runs next may offer buffers that let this block's last product prepare
             # its first norm
             tgt = None
@@ -130,16 +156,18 @@ class DecoderModel:
                 observer(i + 1, resid + delta.float() if isinstance(delta, torch.Tensor) else resid.clone())
         return resid, delta
 
-    def forward(self, batch, caches: Sequence[Optional[LayerCache]], observer=None) -> torch.Tensor:
+    def forward(self, batch, caches: Sequence[Optional[LayerCache]], observer=None, input_states=None) -> torch.Tensor:
         """Logits [len(batch.logit_rows), vocab] in float32 for the step's tokens.
 
         The head runs on the wanted rows only (the reference computes all rows of
         a prompt and keeps the last, crates/cuda/src/engine.rs:5685-5720)."""
-        resid, delta = self.forward_layers(batch, caches, observer)
+        resid, delta = self.forward_layers(batch, caches, observer, input_states)
         if delta is not None and not isinstance(delta, torch.Tensor):
             delta = None               # a filled norm target: the sum is already in the stream
         xn = self.final_norm.add_norm(resid, delta, rows=batch.logit_rows)
         logits = torch.empty((batch.num_logit_rows, self.spec.vocab_size), dtype=torch.float32,
                              device=self.device)
         kernels.current().linear(xn, self.head, logits)
+        if self.spec.logit_softcap > 0.0:
+            kernels.current().tanh_cap(logits, self.spec.logit_softcap)
         return logits

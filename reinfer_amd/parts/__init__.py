@@ -1,7 +1,8 @@
 from .base import KVNeed, LayerCache, PagedNeed, StateNeed
-from .registry import (lookup, register_block, register_feed_forward, register_mixer, register_norm,
-                       register_position)
-from . import attention, block, feed_forward, norm, position  # noqa: F401  (register the parts)
+from .registry import (lookup, register_block, register_feed_forward, register_input, register_mixer,
+                       register_norm, register_position)
+from . import (attention, block, feed_forward, inputs, latent_attention, moe, norm,  # noqa: F401  (register the parts)
+               position)
 
 __all__ = ["KVNeed", "LayerCache", "PagedNeed", "StateNeed", "lookup", "register_block", "register_feed_forward",
-           "register_mixer", "register_norm", "register_position"]
+           "register_input", "register_mixer", "register_norm", "register_position"]

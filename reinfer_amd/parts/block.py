@@ -99,3 +99,69 @@ class PreNormBlock:
         if not (getattr(producer, "emits_for_norm", False) and hasattr(norm, "emit_target")):
             return None
         return norm.emit_target(resid, getattr(consumer, "takes_row_scaled", False))
+
+
+@register_block("parallel")
+class ParallelBlock:
+    """h = norm(x); x += mixer(h) + ffn(h): one norm, and both parts read its output. A block without a
+    feed-forward (``spec.ffn`` None) is x += mixer(norm(x)). The sums are float: a part that can add its last
+    product into the stream does so, any other addend goes through the stream-add kernel or, the last one,
+    back to the caller, whose next norm adds it."""
+
+    @classmethod
+    def declare_params(cls, spec: BlockSpec) -> List[ParamDecl]:
+        p = spec.prefix
+        out = lookup("norm", spec.mixer_norm.kind).declare_params(spec.mixer_norm, p + spec.mixer_norm_name)
+        out += lookup("mixer", spec.mixer.kind).declare_params(spec.mixer, p + spec.mixer_prefix)
+        if spec.ffn is not None:
+            out += lookup("feed_forward", spec.ffn.kind).declare_params(spec.ffn, p + spec.ffn_prefix)
+        return out
+
+    def __init__(self, spec: BlockSpec, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
+                 device: torch.device):
+        missing = [n for n in ("mixer", "mixer_norm") if getattr(spec, n) is None]
+        if missing:
+            raise ValueError(f"a parallel block is made of one norm, a mixer and at most a feed-forward; "
+                             f"block {spec.prefix!r} names no {', '.join(missing)}")
+        p = spec.prefix
+        self.spec = spec
+        self.norm = lookup("norm", spec.mixer_norm.kind)(spec.mixer_norm, weights, p + spec.mixer_norm_name,
+                                                         dtype, device)
+        self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, weights, p + spec.mixer_prefix, dtype, device)
+        self.ffn = None
+        if spec.ffn is not None:
+            self.ffn = lookup("feed_forward", spec.ffn.kind)(spec.ffn, weights, p + spec.ffn_prefix, dtype, device)
+
+    @property
+    def graph_safe(self) -> bool:
+        return bool(getattr(self.mixer, "graph_safe", False)
+                    and (self.ffn is None or getattr(self.ffn, "graph_safe", False)))
+
+    def cache_need(self):
+        return self.mixer.cache_need() if hasattr(self.mixer, "cache_need") else None
+
+    def parts(self):
+        return tuple(p for p in (self.norm, self.mixer, self.ffn) if p is not None)
+
+    def forward(self, resid: torch.Tensor, delta, batch, cache: Optional[LayerCache]):
+        from .. import kernels
+        if not isinstance(delta, torch.Tensor) and delta is not None:
+            delta = None               # a filled norm target: the sum is already in the stream
+        h = self.norm.add_norm(resid, delta)          # the stream now holds everything before this block
+        addends = []
+        if getattr(self.mixer, "adds_in_place", False):
+            a = self.mixer.forward(h, batch, cache, resid=resid)
+        else:
+            a = self.mixer.forward(h, batch, cache)
+        if a is not None:
+            addends.append(a)
+        if self.ffn is not None:
+            if getattr(self.ffn, "adds_in_place", False):
+                b = self.ffn.forward(h, batch, resid=resid)
+            else:
+                b = self.ffn.forward(h, batch)
+            if b is not None:
+                addends.append(b)
+        for a in addends[:-1]:
+            kernels.current().stream_add(resid, a)
+        return addends[-1] if addends else None

@@ -1,0 +1,128 @@
+"""Attention over a cached low-rank latent, inside an optional sliding window.
+
+With h the mixer's input, per token: q = W_q h (heads of [head_dim unrotated | rot_width rotated]),
+(c_raw | kr) = W_dkv h, c = rms(c_raw) * w_c. Head a has keys W_uk,a c and values W_uv,a c, one rotated key
+part kr for all heads, score scale * (q_a . k_a + rot(qr_a) . rot(kr)), softmax over the window, and the
+concatenated heads, times sigmoid(W_g h) where the mixer is gated, go through W_o.
+
+Only c and the rotated key part are cached. Since a head's keys and values are linear in c,
+
+    q_a . (W_uk,a c) = (W_uk,a^T q_a) . c        and        sum_j p_j W_uv,a c_j = W_uv,a (sum_j p_j c_j),
+
+the attention itself runs over the cached rows [c | rot(kr)] as ONE shared KV head of size
+Dp = rank + rot_width (rounded up to the cache's tile of 16) for all query heads, through the same paged
+kernels as grouped-query attention: queries [W_uk,a^T q_a | rot(qr_a)], values the same rows (the columns
+behind ``rank`` of the result are not used). What is new here are the kernel that norms, rotates and writes
+the cache row (``latent_prep``) and the products head by head before and after (``head_linear``).
+q, the latent and the gate come from one fused product.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import kernels
+from ..config.schema import MixerSpec
+from ..weights import VECTOR, ParamDecl
+from .base import KVNeed, LayerCache
+from .registry import lookup, register_mixer
+
+
+def _round16(n: int) -> int:
+    return -(-n // 16) * 16
+
+
+@register_mixer("latent_attention")
+class LatentAttention:
+    graph_safe = True       # no host-side state: a decode step with it can be captured
+    adds_in_place = True    # forward(..., resid=) may add the output projection into the stream
+
+    @classmethod
+    def declare_params(cls, spec: MixerSpec, prefix: str) -> List[ParamDecl]:
+        p = spec.params
+        H, D, R = spec.num_heads, spec.head_dim, p.rot_width
+        out = [ParamDecl(prefix + "q", (H * (D + R), spec.hidden)),
+               ParamDecl(prefix + "dkv", (p.rank + R, spec.hidden)),
+               ParamDecl(prefix + "dkv.norm", (p.rank,), init="norm", role=VECTOR),
+               ParamDecl(prefix + "uk", (H * D, p.rank)),
+               ParamDecl(prefix + "uv", (H * p.value_dim, p.rank))]
+        if p.gated:
+            out.append(ParamDecl(prefix + "g", (H * p.value_dim, spec.hidden)))
+        out.append(ParamDecl(prefix + "o", (spec.hidden, H * p.value_dim)))
+        return out
+
+    def __init__(self, spec: MixerSpec, weights: Dict[str, torch.Tensor], prefix: str,
+                 dtype: torch.dtype, device: torch.device):
+        p = spec.params
+        if p is None:
+            raise ValueError("latent_attention: the mixer's sizes come in MixerSpec.params (LatentAttentionSpec)")
+        self.spec = spec
+        self.dtype = dtype
+        self.num_heads, self.head_dim = int(spec.num_heads), int(spec.head_dim)
+        self.rank, self.rot_width, self.value_dim = int(p.rank), int(p.rot_width), int(p.value_dim)
+        self.gated = bool(p.gated)
+        self.eps = float(p.norm_eps)
+        self.scale = float(spec.scale)
+        self.window = int(spec.window)
+        self.cache_dim = _round16(self.rank + self.rot_width)
+        H, D, R, Dv = self.num_heads, self.head_dim, self.rot_width, self.value_dim
+        # one product for everything that reads the mixer's input: rows of q, of the latent, of the gate
+        rows = [weights[prefix + "q"], weights[prefix + "dkv"]]
+        self.q_off, self.dkv_off = 0, H * (D + R)
+        self.gate_off = self.dkv_off + self.rank + R
+        if self.gated:
+            rows.append(weights[prefix + "g"])
+        self.proj_width = sum(int(w.shape[0]) for w in rows)
+        pad = (-self.proj_width) % 8            # rows of 16-byte pieces for the kernels that read them
+        if pad:
+            rows.append(torch.zeros((pad, spec.hidden), dtype=rows[0].dtype, device=rows[0].device))
+        self.proj_width += pad
+        self.w_in = torch.cat(rows, dim=0).contiguous()
+        self.c_norm = weights[prefix + "dkv.norm"]
+        # head products, [heads, K, N] with N contiguous: queries through the key matrices, W_uk[a, d, r] as stored;
+        # results through the value matrices, W_uv[a, v, r] transposed to [a, r, v]
+        self.w_absorb = weights[prefix + "uk"].view(H, D, self.rank).contiguous()
+        self.w_values = weights[prefix + "uv"].view(H, Dv, self.rank).transpose(1, 2).contiguous()
+        self.w_o = weights[prefix + "o"]
+        self.position = lookup("position", spec.position.kind)(spec.position, device)
+        if self.position.rotary_dim > R:
+            raise ValueError("the rotated width cannot exceed the rotated part of a head")
+
+    def cache_need(self) -> KVNeed:
+        return KVNeed(1, self.cache_dim, self.window)
+
+    def plan_captured_step(self, batch, num_rows: int, ctx_cap: int) -> None:
+        hook = getattr(kernels.current(), "plan_captured_step", None)
+        if hook is not None:
+            hook(batch, num_rows, ctx_cap)
+
+    def forward(self, x, batch, cache: LayerCache, resid: Optional[torch.Tensor] = None):
+        ops = kernels.current()
+        T = x.shape[0]
+        H, D, Dv, Dp = self.num_heads, self.head_dim, self.value_dim, self.cache_dim
+        slots = batch.slots[cache.group] if cache.writes else batch.no_slots
+        proj = torch.empty((T, self.proj_width), dtype=self.dtype, device=x.device)
+        ops.linear(x, self.w_in, proj)
+        q_lat = torch.empty((T, H, Dp), dtype=self.dtype, device=x.device)
+        ops.latent_prep(proj, self.q_off, self.dkv_off, self.c_norm, self.eps, batch.positions,
+                        self.position.inv_freq, self.position.rotary_dim, self.rot_width, self.rank, H, D,
+                        q_lat, slots, cache.k, cache.v)
+        q_rows = q_lat.view(T, H * Dp)
+        if D > 0:
+            ops.head_linear(proj[:, self.q_off:], D + self.rot_width, self.w_absorb, q_rows, Dp)
+        else:
+            q_lat[:, :, :self.rank].zero_()
+        o_lat = torch.empty((T, H * Dp), dtype=self.dtype, device=x.device)
+        ops.attention(q_rows, H * Dp, o_lat, cache.k, cache.v, batch, H, 1, Dp, self.scale, self.window,
+                      cache.group)
+        heads = torch.empty((T, H * Dv), dtype=self.dtype, device=x.device)
+        ops.head_linear(o_lat, Dp, self.w_values, heads, Dv,
+                        gate=proj[:, self.gate_off:self.gate_off + H * Dv] if self.gated else None)
+        can_add = getattr(ops, "can_accumulate", None)
+        if resid is not None and can_add and can_add(heads, self.w_o):
+            ops.linear_skinny(heads, self.w_o, resid, accumulate=True)
+            return None
+        out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
+        ops.linear(heads, self.w_o, out)
+        return out

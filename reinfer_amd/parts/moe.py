@@ -1,0 +1,71 @@
+"""Mixture-of-experts feed-forward: a router picks ``top`` of ``experts`` small feed-forward layers a token.
+
+Router logits z = W_r h in float; the ``top`` largest are chosen and weighted by the softmax over the chosen
+logits alone; an expert is W_down act(W_up h) with act = relu squared, no bias; the output is the weighted
+sum of the chosen experts' outputs.
+
+The experts' up projections are laid side by side as one [experts * ff, width] matrix and their down
+projections as one [width, experts * ff] matrix. A step computes every expert's up projection in one product,
+applies the activation and the routing weight in one kernel (0 for experts a token did not choose), and one
+product with the down matrix is then the weighted sum: with few experts of which a good share is chosen, two
+dense products at the matrix cores' rate cost less than gathering tokens by expert would.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import kernels
+from ..config.schema import FeedForwardSpec
+from ..weights import ParamDecl
+from .registry import register_feed_forward
+
+
+@register_feed_forward("moe")
+class MixtureOfExperts:
+    graph_safe = True       # routing stays on the device: a decode step with it can be captured
+    adds_in_place = True    # forward(..., resid=) may add the down projection into the stream
+
+    @classmethod
+    def declare_params(cls, spec: FeedForwardSpec, prefix: str) -> List[ParamDecl]:
+        p = spec.params
+        out = []
+        for e in range(p.experts):
+            out += [ParamDecl(f"{prefix}e{e}.up", (spec.intermediate, spec.hidden)),
+                    ParamDecl(f"{prefix}e{e}.down", (spec.hidden, spec.intermediate))]
+        out.append(ParamDecl(prefix + "router", (p.experts, spec.hidden)))
+        return out
+
+    def __init__(self, spec: FeedForwardSpec, weights: Dict[str, torch.Tensor], prefix: str,
+                 dtype: torch.dtype, device: torch.device):
+        p = spec.params
+        if p is None:
+            raise ValueError("moe: the routing comes in FeedForwardSpec.params (MoESpec)")
+        if p.activation != "relu2" or p.weights != "softmax_chosen":
+            raise ValueError(f"moe: activation {p.activation!r} with weights {p.weights!r} is not built")
+        self.spec = spec
+        self.dtype = dtype
+        self.experts, self.top, self.ff = int(p.experts), int(p.top), int(spec.intermediate)
+        self.w_up = torch.cat([weights[f"{prefix}e{e}.up"] for e in range(self.experts)], dim=0).contiguous()
+        self.w_down = torch.cat([weights[f"{prefix}e{e}.down"] for e in range(self.experts)], dim=1).contiguous()
+        self.router = weights[prefix + "router"].to(torch.float32).contiguous()      # logits are float
+
+    def forward(self, x, batch, resid: Optional[torch.Tensor] = None):
+        ops = kernels.current()
+        T = x.shape[0]
+        n = self.experts * self.ff
+        ids = torch.empty((T, self.top), dtype=torch.int32, device=x.device)
+        weights = torch.empty((T, self.top), dtype=torch.float32, device=x.device)
+        ops.moe_route(x, self.router, self.top, ids, weights)
+        up = torch.empty((T, n), dtype=self.dtype, device=x.device)
+        ops.linear(x, self.w_up, up)
+        act = torch.empty((T, n), dtype=self.dtype, device=x.device)
+        ops.moe_relu2_scale(up, act, ids, weights, self.experts, self.ff)
+        can_add = getattr(ops, "can_accumulate", None)
+        if resid is not None and can_add and can_add(act, self.w_down):
+            ops.linear_skinny(act, self.w_down, resid, accumulate=True)
+            return None
+        out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
+        ops.linear(act, self.w_down, out)
+        return out

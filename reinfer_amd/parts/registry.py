@@ -14,7 +14,7 @@ from __future__ import annotations
 from typing import Any, Callable, Dict
 
 _REGISTRIES: Dict[str, Dict[str, Any]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {},
-                                          "block": {}}
+                                          "block": {}, "input": {}}
 
 
 def _register(kind_of_part: str, name: str, cls: Any = None):
@@ -42,6 +42,10 @@ def register_position(name: str, cls: Any = None):
 
 def register_block(name: str, cls: Any = None):
     return _register("block", name, cls)
+
+
+def register_input(name: str, cls: Any = None):
+    return _register("input", name, cls)
 
 
 def lookup(kind_of_part: str, name: str):

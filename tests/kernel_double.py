@@ -84,6 +84,96 @@ class KernelDouble:
             kflat[s // bs][:, k_index(s % bs, e, d)] = k[t].to(kcache.dtype)
             vflat[s // bs][:, v_index(s % bs, e, d)] = v[t].to(vcache.dtype)
 
+    # ---- around the stream
+    def pair_hash_add(self, resid, table, batch, last_token, buckets, mul_prev, mul_cur):
+        ids, pos = batch.token_ids.tolist(), batch.positions.tolist()
+        cu, seq_of = batch.cu_tokens.tolist(), batch.seq_of_token.tolist()
+        for t in range(batch.num_tokens):
+            i = seq_of[t]
+            slot = int(batch.state_slots[i])
+            prev = -1
+            if t != cu[i]:
+                prev = ids[t - 1]
+            else:
+                if pos[t] > 0 and slot >= 0:
+                    prev = int(last_token[slot])
+                if slot >= 0:
+                    last_token[slot] = ids[cu[i + 1] - 1]
+            row = buckets if (pos[t] == 0 or prev < 0) else (prev * mul_prev + ids[t] * mul_cur) % buckets
+            resid[t] += table[row].float()
+
+    def stream_add(self, resid, delta=None, other=None, vec=None):
+        if delta is not None:
+            resid.add_(delta.float())
+        if other is not None:
+            resid.add_(other)
+        if vec is not None:
+            resid.add_(vec.float())
+
+    def tanh_cap(self, logits, cap):
+        logits.copy_(cap * torch.tanh(logits / cap))
+
+    # ---- latent attention
+    def latent_prep(self, proj, q_off, dkv_off, c_weight, eps, positions, inv_freq, rot_dims, rot_width, rank,
+                    num_heads, head_dim, q_lat, slots, kcache, vcache):
+        T = proj.shape[0]
+        Dp = q_lat.shape[2]
+        half = rot_dims // 2
+        ang = positions.float()[:, None] * inv_freq[:half].float()[None, :] if half else None
+
+        def rot(x):                      # [T, ..., rot_width]
+            if not half:
+                return x
+            shape = [T] + [1] * (x.dim() - 2) + [half]
+            c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+            out = x.clone()
+            a, b = x[..., :half], x[..., half:rot_dims]
+            out[..., :half] = a * c - b * s
+            out[..., half:rot_dims] = b * c + a * s
+            return out
+
+        p = proj.float()
+        craw = p[:, dkv_off:dkv_off + rank]
+        c = craw * torch.rsqrt((craw * craw).mean(dim=-1, keepdim=True) + eps) * c_weight.float()
+        kr = rot(p[:, dkv_off + rank:dkv_off + rank + rot_width])
+        row = torch.zeros((T, Dp))
+        row[:, :rank] = c
+        row[:, rank:rank + rot_width] = kr
+        q = p[:, q_off:q_off + num_heads * (head_dim + rot_width)].view(T, num_heads, head_dim + rot_width)
+        q_lat[:, :, rank:] = 0
+        q_lat[:, :, rank:rank + rot_width] = rot(q[:, :, head_dim:]).to(q_lat.dtype)
+        bs = kcache.shape[2] * 16
+        kflat, vflat = kcache.view(kcache.shape[0], 1, -1), vcache.view(vcache.shape[0], 1, -1)
+        e = torch.arange(Dp)
+        for t in range(T):
+            s = int(slots[t])
+            if s < 0:
+                continue
+            kflat[s // bs][:, k_index(s % bs, e, Dp)] = row[t].to(kcache.dtype)
+            vflat[s // bs][:, v_index(s % bs, e, Dp)] = row[t].to(vcache.dtype)
+
+    def head_linear(self, x, x_head, weight, out, o_head, gate=None):
+        H, K, N = weight.shape
+        for h in range(H):
+            y = x[:, h * x_head:h * x_head + K].float() @ weight[h].float()
+            if gate is not None:
+                y = y * torch.sigmoid(gate[:, h * N:(h + 1) * N].float())
+            out[:, h * o_head:h * o_head + N] = y.to(out.dtype)
+
+    # ---- mixture of experts
+    def moe_route(self, x, router, top, ids, weights):
+        z = x.float() @ router.float().T
+        val, idx = torch.topk(z, top, dim=-1)
+        ids.copy_(idx.to(torch.int32))
+        weights.copy_(torch.softmax(val, dim=-1))
+
+    def moe_relu2_scale(self, up, act, ids, weights, experts, ff):
+        T = up.shape[0]
+        gate = torch.zeros((T, experts))
+        gate.scatter_(1, ids.long(), weights)
+        u = torch.relu(up.float()).view(T, experts, ff)
+        act.copy_((gate[:, :, None] * u * u).view(T, experts * ff).to(act.dtype))
+
     GATE_GROUP = 8
 
     def silu_mul(self, gate_up, out, group=0):
