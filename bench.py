@@ -356,6 +356,113 @@ def serve_run(args, raw, shape_name: str) -> int:
     return 0
 
 
+# ---------------------------------------------------------------------------------------------------
+# --design puresun: the Puresun design beside the Qwen3 dense decoder at equal size
+# ---------------------------------------------------------------------------------------------------
+def _puresun_raw(width, heads, layers, loop, experts, top, ff, window, vocab):
+    mixer = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5,
+             "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 64}}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    raw = {"architecture": "Puresun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+           "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+           "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
+    if loop:
+        raw["loop"] = {"start": 0, "stop": loop[0], "times": loop[1]}
+    return raw
+
+
+# (name, Puresun configuration, its Qwen3 twin): as many layer runs, the same width, heads and window, a dense
+# feed-forward with the parameters a token's chosen experts have (3 h I = 2 h ff top)
+def design_sizes():
+    out = []
+    for name, width, heads, layers, loop, experts, top, ff in (("w2048", 2048, 16, 8, (4, 2), 8, 2, 2048),
+                                                               ("w4096", 4096, 16, 6, (2, 2), 16, 4, 1536)):
+        vocab, window = 32768, 1024
+        runs = layers + (loop[0] * (loop[1] - 1) if loop else 0)
+        inter = -(-(2 * ff * top // 3) // 64) * 64
+        twin = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "num_hidden_layers": runs,
+                "hidden_size": width, "num_attention_heads": heads, "num_key_value_heads": 4, "head_dim": 128,
+                "intermediate_size": inter, "vocab_size": vocab, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+                "tie_word_embeddings": False, "max_position_embeddings": 8192, "attention_bias": False,
+                "sliding_window": window, "use_sliding_window": True, "max_window_layers": 0}
+        out.append((name, _puresun_raw(width, heads, layers, loop, experts, top, ff, window, vocab), twin, vocab))
+    return out
+
+
+def design_run(args) -> int:
+    """Prefill and decode throughput of Puresun and of its Qwen3 twin at each size, and the GPU time of a
+    2,048-token prompt step and of a decode step at batch 8 by kernel class with each class's share of its
+    roofline (weight bytes over 8 TB/s or flops over 2.5 PFLOP/s, whichever is longer). One JSON line."""
+    import gc
+    import torch
+    from reinfer_amd import kernels
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.engine import LLMEngine, StepEntry
+    from reinfer_amd.kernels.profile import TimedKernels
+    from reinfer_amd.sampling import SamplingParams
+
+    def classes(engine, vocab, n_tokens, batch, ctx):
+        """kernel class -> ms, share of its roofline, for one eager step of ``batch`` requests bringing
+        ``n_tokens`` each behind ``ctx`` cached tokens."""
+        runner = engine.runner
+        g = torch.Generator().manual_seed(3)
+        rids = [f"p{i}" for i in range(batch)]
+        for r in rids:
+            runner.add_request(r)
+            if ctx:
+                runner.step([StepEntry(r, torch.randint(0, vocab, (ctx,), generator=g).tolist(), [])])
+        timed = TimedKernels(kernels.current())
+        graphs, runner.graphs = runner.graphs, None
+        try:
+            with kernels.use(timed):
+                timed.hold_back(25.0, engine.device)
+                runner.step([StepEntry(r, torch.randint(0, vocab, (n_tokens,), generator=g).tolist(), [n_tokens - 1])
+                             for r in rids])
+            rows = timed.report()
+        finally:
+            runner.graphs = graphs
+            for r in rids:
+                runner.free_request(r)
+        out = {}
+        for label, row in sorted(rows.items(), key=lambda kv: -kv[1]["ms"]):
+            roof = max(row["bytes"] / HBM_PEAK, row["flops"] / MFMA_PEAK["bf16"]) * 1e3
+            out[label] = {"ms": round(row["ms"], 4), "calls": row["calls"],
+                          "of_roofline": round(roof / row["ms"], 3) if row["ms"] > 0 and roof > 0 else None}
+        return out
+
+    results = {}
+    for name, p_raw, q_raw, vocab in design_sizes():
+        for which, raw in (("puresun", p_raw), ("qwen3", q_raw)):
+            cfg = config_from_dict(raw)
+            log(f"{name} {which}: building ...")
+            engine = LLMEngine(config=cfg, seed=args.seed, dtype=args.dtype, block_size=16,
+                               num_blocks=64 * 160 + 512, max_num_seqs=64, max_num_batched_tokens=2048,
+                               max_model_len=4096)
+            fake = {"vocab_size": vocab}
+            rec = {}
+            ms = prefill_run(engine, fake, 2048, 3, args.seed + 1)
+            rec["prefill_2048_tok_s"] = round(2048 / (ms * 1e-3), 1)
+            for b in (8, 64):
+                dms, ctx = decode_run(engine, fake, b, 1536, 32, 8, args.seed + 2 + b, 2048)
+                rec[f"decode_b{b}_tok_s"] = round(b / (dms * 1e-3), 1)
+                rec[f"decode_b{b}_ms"] = round(dms, 3)
+            rec["prefill_2048_classes"] = classes(engine, vocab, 2048, 1, 0)
+            rec["decode_b8_classes"] = classes(engine, vocab, 1, 8, 1536)
+            log(f"{name} {which}: prefill {rec['prefill_2048_tok_s']:.0f} tok/s, decode batch 8 "
+                f"{rec['decode_b8_tok_s']:.0f} tok/s ({rec['decode_b8_ms']} ms), batch 64 {rec['decode_b64_tok_s']:.0f} tok/s "
+                f"({rec['decode_b64_ms']} ms)")
+            for step in ("prefill_2048_classes", "decode_b8_classes"):
+                for label, row in rec[step].items():
+                    log(f"    {step[:-8]:13s} {label:40s} {row['ms']:8.3f} ms  {row['calls']:4d} calls  of roofline {row['of_roofline']}")
+            results.setdefault(name, {})[which] = rec
+            del engine
+            gc.collect()
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "puresun_beside_qwen3", "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic", "n_gpus": 1, "sizes": results}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -376,6 +483,8 @@ def main() -> int:
     ap.add_argument("--max-model-len", type=int, default=None, metavar="N",
                     help="context length (default: the shape's: 4096 at 8b, 8192 at 4b, 16384 at 32b)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the Qwen3-8B shape)")
+    ap.add_argument("--design", default=None, choices=["puresun"],
+                    help="instead of the default measurement: this design beside the Qwen3 decoder at equal sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -390,6 +499,8 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3
     kernels.current()
+    if args.design:
+        return design_run(args)
     shape_name, shape = SHAPES[args.shape]
     raw = dict(shape)
     full_layers = raw["num_hidden_layers"]

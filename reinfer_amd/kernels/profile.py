@@ -28,6 +28,10 @@ _ROWS = {"embed": "embedding", "add_rmsnorm": "norm", "silu_mul": "gate", "sampl
 _QK = {"qk_norm_rope_cache", "qk_norm_rope_cache_ranges"}
 _ATTN = {"attention", "attention_plain", "attention_decode", "attention_prefill"}
 _LINEAR = {"linear", "linear_plain", "linear_skinny", "gated_linear", "linear_ranges"}
+# kernels of further mechanisms, each a class of its own
+_OTHER = {"latent_prep": "latent norm + rotation + cache write", "head_linear": "products head by head",
+          "moe_route": "router", "moe_relu2_scale": "expert activation", "stream_add": "stream add",
+          "pair_hash_add": "embedding", "tanh_cap": "logit cap"}
 
 
 class TimedKernels:
@@ -36,7 +40,7 @@ class TimedKernels:
     def __init__(self, inner):
         self._inner = inner
         self._names: Dict[int, str] = {}
-        self._spans: List[Tuple[str, torch.cuda.Event, torch.cuda.Event]] = []
+        self._spans: List[Tuple[str, torch.cuda.Event, torch.cuda.Event, int, int]] = []
         self._filler: Optional[torch.Tensor] = None
         self.name = getattr(inner, "name", "timed")
 
@@ -50,6 +54,8 @@ class TimedKernels:
             return "head norm + rotation + cache write"
         if method in _ATTN:
             return "attention"
+        if method in _OTHER:
+            return _OTHER[method]
         if method in _LINEAR:
             w = args[1] if len(args) > 1 else kwargs.get("weight")
             role = self._names.get(w.data_ptr()) if isinstance(w, torch.Tensor) else None
@@ -58,7 +64,8 @@ class TimedKernels:
 
     def __getattr__(self, attr: str) -> Any:
         target = getattr(self._inner, attr)
-        if not callable(target) or not (attr in _ROWS or attr in _QK or attr in _ATTN or attr in _LINEAR):
+        if not callable(target) or not (attr in _ROWS or attr in _QK or attr in _ATTN or attr in _LINEAR
+                                        or attr in _OTHER):
             return target
 
         def timed_call(*args, **kwargs):
@@ -66,7 +73,17 @@ class TimedKernels:
             e0.record()
             out = target(*args, **kwargs)
             e1.record()
-            self._spans.append((self._label(attr, args, kwargs), e0, e1))
+            # what a product must read (its weight) and compute, for pricing the class against the machine
+            nbytes = flops = 0
+            w = None
+            if attr in _LINEAR:
+                w = args[1] if len(args) > 1 else kwargs.get("weight")
+            elif attr == "head_linear":
+                w = args[2] if len(args) > 2 else kwargs.get("weight")
+            if isinstance(w, torch.Tensor) and isinstance(args[0], torch.Tensor):
+                nbytes = w.numel() * w.element_size()
+                flops = 2 * args[0].shape[0] * w.numel()
+            self._spans.append((self._label(attr, args, kwargs), e0, e1, nbytes, flops))
             return out
         return timed_call
 
@@ -84,7 +101,8 @@ class TimedKernels:
                          torch.cuda.current_stream().cuda_stream)
 
     def report(self) -> Dict[str, Dict[str, float]]:
-        """class -> {"calls", "ms"}; clears what was recorded."""
+        """class -> {"calls", "ms", "bytes", "flops"} (the last two for products: weight bytes read, flops);
+        clears what was recorded."""
         pairs = []
         for _ in range(16):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -94,9 +112,11 @@ class TimedKernels:
         torch.cuda.synchronize()
         empty = sorted(a.elapsed_time(b) for a, b in pairs)[len(pairs) // 2]
         out: Dict[str, Dict[str, float]] = {}
-        for label, e0, e1 in self._spans:
-            row = out.setdefault(label, {"calls": 0, "ms": 0.0})
+        for label, e0, e1, nbytes, flops in self._spans:
+            row = out.setdefault(label, {"calls": 0, "ms": 0.0, "bytes": 0, "flops": 0})
             row["calls"] += 1
             row["ms"] += max(0.0, e0.elapsed_time(e1) - empty)
+            row["bytes"] += nbytes
+            row["flops"] += flops
         self._spans = []
         return out

@@ -98,17 +98,26 @@ def latent_attention(h: torch.Tensor, w: Mapping[str, torch.Tensor], pre: str, m
     return o @ w[pre + "o"].T
 
 
+def route(h: torch.Tensor, router: torch.Tensor, top: int):
+    """(chosen experts [n, top] in falling order of their logits, their weights [n, top])."""
+    z = h @ router.T
+    val, idx = torch.topk(z, top, dim=-1)
+    return idx, torch.softmax(val, dim=-1)
+
+
+def expert(h: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
+    return (torch.relu(h @ up.T) ** 2) @ down.T
+
+
 def moe_feed_forward(h: torch.Tensor, w: Mapping[str, torch.Tensor], pre: str, f: Mapping) -> torch.Tensor:
     E, top = int(f["router"]["experts"]), int(f["router"]["top"])
-    z = h.float() @ w[pre + "router"].float().T if h.dtype != torch.float64 else h @ w[pre + "router"].T
-    val, idx = torch.topk(z, top, dim=-1)
-    p = torch.softmax(val, dim=-1).to(h.dtype)
+    idx, p = route(h, w[pre + "router"], top)
     out = torch.zeros_like(h)
-    for t in range(h.shape[0]):
-        for j in range(top):
-            e = int(idx[t, j])
-            a = torch.relu(h[t] @ w[f"{pre}e{e}.up"].T) ** 2
-            out[t] += p[t, j] * (a @ w[f"{pre}e{e}.down"].T)
+    for e in range(E):
+        share = (p * (idx == e)).sum(dim=-1, keepdim=True)          # 0 where the token did not choose e
+        rows = share[:, 0] > 0
+        if rows.any():
+            out[rows] += share[rows] * expert(h[rows], w[f"{pre}e{e}.up"], w[f"{pre}e{e}.down"])
     return out
 
 
@@ -155,3 +164,13 @@ def forward(cfg: Mapping, w: Mapping[str, torch.Tensor], tokens: Sequence[int], 
     if softcap and cap:
         y = float(cap) * torch.tanh(y / float(cap))
     return y
+
+
+def greedy_generate(cfg: Mapping, w: Mapping[str, torch.Tensor], prompt: Sequence[int], n_new: int) -> List[int]:
+    """The first maximum of the last position's logits, n_new times, the whole sequence recomputed each time."""
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        t = int(torch.argmax(forward(cfg, w, toks)[-1]))
+        out.append(t)
+        toks.append(t)
+    return out

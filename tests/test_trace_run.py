@@ -198,3 +198,42 @@ def test_trace_run_checks_start_against_what_the_cache_holds(tmp_path):
         assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == ["done 0"]
         assert (out / "0.f32").exists() and not (out / "1.f32").exists()
         assert "start" in proc.stderr and repr(bad["id"]) in proc.stderr
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("A16", "bfloat16")])
+def test_trace_run_puresun(tmp_path, which, dtype):
+    """Another architecture through the same program: the model class comes from config.json. Portions beside
+    single tokens, a request left out of a step, state slots and blocks used again."""
+    import plain_puresun
+    import puresun_helpers as ph
+    from test_puresun_engine import TOL as PTOL
+    folder = ph.make_folder(tmp_path, which, dtype)
+    raw, weights = ph.read_folder(folder)
+    V = raw["vocab"]
+    seqs = {"a": random_tokens(70, V, 1), "b": random_tokens(41, V, 2), "c": random_tokens(50, V, 3)}
+    refs = {r: plain_puresun.forward(raw, weights, t).float() for r, t in seqs.items()}
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": seqs["a"][:33], "want": [0, 32]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": seqs["a"][33:69], "want": list(range(36))},
+                                {"id": "b", "tokens": seqs["b"][:2], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": seqs["b"][2:40], "want": [37]}], "end": []},
+        {"step": 3, "entries": [{"id": "b", "tokens": seqs["b"][40:41], "want": [0]},
+                                {"id": "a", "tokens": seqs["a"][69:70], "want": [0]}], "end": ["a", "b"]},
+        {"step": 4, "entries": [{"id": "c", "tokens": seqs["c"][:49], "want": [5]}], "end": []},
+        {"step": 5, "entries": [{"id": "c", "tokens": seqs["c"][49:50], "want": [0]}], "end": ["c"]},
+    ]
+    out = tmp_path / f"out_{dtype}"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", str(out), "--max-tokens", "128"],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(6)]
+    fed = {r: 0 for r in seqs}
+    for s in steps:
+        want_rows = []
+        for e in s["entries"]:
+            want_rows += [refs[e["id"]][fed[e["id"]] + w] for w in e["want"]]
+            fed[e["id"]] += len(e["tokens"])
+        got = torch.from_numpy(np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(len(want_rows), V))
+        assert rel_err(got, torch.stack(want_rows)) < PTOL[dtype]
