@@ -443,7 +443,7 @@ def design_run(args) -> int:
             ms = prefill_run(engine, fake, 2048, 3, args.seed + 1)
             rec["prefill_2048_tok_s"] = round(2048 / (ms * 1e-3), 1)
             for b in (8, 64):
-                dms, ctx = decode_run(engine, fake, b, 1536, 32, 8, args.seed + 2 + b, 2048)
+                dms, ctx = decode_run(engine, fake, b, 1536, 32, 8, args.seed + 2 + b, b + 32 + 8 + 16)
                 rec[f"decode_b{b}_tok_s"] = round(b / (dms * 1e-3), 1)
                 rec[f"decode_b{b}_ms"] = round(dms, 3)
             rec["prefill_2048_classes"] = classes(engine, vocab, 2048, 1, 0)

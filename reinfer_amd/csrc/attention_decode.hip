@@ -411,8 +411,10 @@ static int fd_resident_workgroups(int variant, int waves, size_t lds) {
 extern "C" int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_size) {
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return 0;
   const int G = Hq / Hkv;
+  // the waves of a workgroup add their partial results through LDS: the small form (4 waves) must fit
+  const size_t lds = (size_t)4 * G * (d + 2) * sizeof(float);
   return (G >= 1 && G <= 16 && d % 16 == 0 && d >= 16 && d <= 256 && block_size > 0 &&
-          block_size % 16 == 0) ? 1 : 0;
+          block_size % 16 == 0 && lds <= 64 * 1024) ? 1 : 0;
 }
 
 // Workgroups of the decode kernel, in its form with `waves` waves a workgroup (4 or 12), that the current

@@ -100,11 +100,71 @@ extern "C" int ra_latent_prep(const void* proj, int act_dtype, int ld, int q_off
 }
 
 // ---------------------------------------------------------------------------
-// Products head by head: out[t, h, n] = sum_k x[t, h, k] * W[h, k, n]   (W: [H, K, N], n contiguous)
+// Products head by head: out[t, h, n] = sum_k x[t, h, k] * W[h, n, k]   (W: [H, N, K], k contiguous)
 // optionally times sigmoid(gate[t, h * N + n]). x, out and gate are rows with strides of their own, a head
-// of x at h * x_head, of out at h * o_head. A workgroup takes 16 tokens of one head: their x in LDS as
-// float [K][16], a thread one output column n at a time, float accumulation.
+// of x at h * x_head, of out at h * o_head.
+//
+// bfloat16 with K, the row strides and the head offsets of x in steps of 8 elements: matrix cores. A wave
+// owns 16 output columns of one head for MT tiles of 16 tokens and walks K in steps of 32; both operands come
+// straight from memory in operand layout (lane (r, g): row r, elements 8g .. 8g + 7 of the step, one 16-byte
+// load), the weights of a head being small enough to stay in the caches while the token tiles pass. The four
+// waves of a workgroup take four column tiles. Lane (r, g) ends with out[token r][column 4g .. 4g + 3].
+// Anything else (float, odd sizes): a plain kernel, 16 tokens of one head a workgroup, x in LDS as float.
 // ---------------------------------------------------------------------------
+template <int MT>
+__global__ void __launch_bounds__(256)
+head_linear_mfma_kernel(const bf16_t* __restrict__ x, int ldx, int x_head, const bf16_t* __restrict__ W,
+                        bf16_t* __restrict__ out, int ldo, int o_head, const bf16_t* __restrict__ gate, int ldg,
+                        int T, int N, int K) {
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE;
+  const int r = lane & 15, g = lane >> 4;
+  const int h = blockIdx.z;
+  const int n0 = (blockIdx.x * 4 + wave) * 16;
+  const int t0 = blockIdx.y * 16 * MT;
+  if (n0 >= N) return;
+  const bf16_t* wrow = W + ((size_t)h * N + (n0 + r < N ? n0 + r : 0)) * K;
+  const bool w_ok = n0 + r < N;
+  const bf16_t* xrow[MT];
+  bool x_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int t = t0 + mt * 16 + r;
+    x_ok[mt] = t < T;
+    xrow[mt] = x + (size_t)(x_ok[mt] ? t : 0) * ldx + (size_t)h * x_head;
+  }
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int k = k0 + g * 8;
+    const bool k_ok = k < K;                          // K is a multiple of 8: a chunk is whole or absent
+    const bf16x8_t a = (w_ok && k_ok) ? *(const bf16x8_t*)(wrow + k) : zero;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const bf16x8_t b = (x_ok[mt] && k_ok) ? *(const bf16x8_t*)(xrow[mt] + k) : zero;
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int t = t0 + mt * 16 + r;
+    if (t >= T) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * g + i;
+      if (n >= N) continue;
+      float v = acc[mt][i];
+      if (gate) {
+        const float gv = to_f32(gate[(size_t)t * ldg + (size_t)h * N + n]);
+        v *= 1.f / (1.f + expf(-gv));
+      }
+      out[(size_t)t * ldo + (size_t)h * o_head + n] = from_f32<bf16_t>(v);
+    }
+  }
+}
+
 #define HL_TOKENS 16
 template <typename TA>
 __global__ void head_linear_kernel(const TA* __restrict__ x, int ldx, int x_head, const TA* __restrict__ W,
@@ -120,12 +180,13 @@ __global__ void head_linear_kernel(const TA* __restrict__ x, int ldx, int x_head
   }
   __syncthreads();
   const TA* Wh = W + (size_t)h * K * N;
-  for (int n = threadIdx.x; n < N; n += blockDim.x) {
+  for (int n = blockIdx.z * blockDim.x + threadIdx.x; n < N; n += gridDim.z * blockDim.x) {
     float acc[HL_TOKENS];
 #pragma unroll
     for (int i = 0; i < HL_TOKENS; ++i) acc[i] = 0.f;
+    const TA* wr = Wh + (size_t)n * K;
     for (int k = 0; k < K; ++k) {
-      const float w = to_f32(Wh[(size_t)k * N + n]);
+      const float w = to_f32(wr[k]);
       const f32x4_t* xr = (const f32x4_t*)(xs + k * HL_TOKENS);
 #pragma unroll
       for (int g = 0; g < HL_TOKENS / 4; ++g) {
@@ -157,12 +218,34 @@ extern "C" int ra_head_linear(const void* x, int ldx, int x_head, const void* W,
   RA_CHECK(ldx >= (H - 1) * x_head + K && ldo >= (H - 1) * o_head + N && x_head >= 0 && o_head >= N,
            "head_linear: rows of %d / %d do not hold %d heads of %d / %d", ldx, ldo, H, K, N);
   RA_CHECK(gate == nullptr || ldg >= H * N, "head_linear: gate rows of %d for %d heads of %d", ldg, H, N);
+  RA_CHECK(H <= 65535, "head_linear: %d heads in one launch", H);
+  if (act_dtype == RA_BF16 && K % 8 == 0 && ldx % 8 == 0 && x_head % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
+      ((uintptr_t)W % 16) == 0) {
+    const int col_groups = (N + 63) / 64;
+    if (n_tokens <= 16) {
+      dim3 grid(col_groups, 1, H);
+      head_linear_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, x_head, (const bf16_t*)W,
+                                                           (bf16_t*)out, ldo, o_head, (const bf16_t*)gate, ldg,
+                                                           n_tokens, N, K);
+    } else {
+      const int tiles = (n_tokens + 63) / 64;
+      RA_CHECK(tiles <= 65535, "head_linear: %d tokens in one launch", n_tokens);
+      dim3 grid(col_groups, tiles, H);
+      head_linear_mfma_kernel<4><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, x_head, (const bf16_t*)W,
+                                                           (bf16_t*)out, ldo, o_head, (const bf16_t*)gate, ldg,
+                                                           n_tokens, N, K);
+    }
+    RA_LAUNCH_CHECK("head_linear");
+    return 0;
+  }
   const size_t lds = (size_t)K * HL_TOKENS * sizeof(float);
   RA_CHECK(lds <= 64 * 1024, "head_linear: K = %d is more than the 1024 a workgroup stages", K);
   const int tiles = (n_tokens + HL_TOKENS - 1) / HL_TOKENS;
   RA_CHECK(tiles <= 65535, "head_linear: %d tokens in one launch", n_tokens);
-  dim3 grid(H, tiles);
   const int threads = N >= 256 ? 256 : ((N + 63) / 64) * 64;
+  // few tokens: the columns of a head are spread over several workgroups as well
+  const int col_groups = tiles * H >= 256 ? 1 : (N + threads - 1) / threads;
+  dim3 grid(H, tiles, col_groups);
   if (act_dtype == RA_F32)
     head_linear_kernel<float><<<grid, threads, lds, stream>>>((const float*)x, ldx, x_head, (const float*)W,
                                                               (float*)out, ldo, o_head, (const float*)gate, ldg,

@@ -193,10 +193,10 @@ int ra_head_linear(const void* x, int ldx, int x_head, const void* W, void* out,
                    const void* gate, int ldg, int act_dtype, int n_tokens, int H, int N, int K, hipStream_t stream);
 
 // ---- mixture of experts (moe.hip) ----
-// float router logits of x [n_tokens, width] against router [experts, width] (float), the `top` (<= 64) largest
-// in falling order into ids [n_tokens, top], their softmax over the chosen alone into weights [n_tokens, top]
-int ra_moe_route(const void* x, int act_dtype, int ldx, const float* router, int experts, int width, int top,
-                 int* ids, float* weights, int n_tokens, hipStream_t stream);
+// the `top` (<= 64) largest of each row of float logits [n_tokens, experts] (row stride ld) in falling order into
+// ids [n_tokens, top] (ties: the lower expert first), their softmax over the chosen alone into weights [n_tokens, top]
+int ra_moe_topk(const float* logits, int ld, int experts, int top, int* ids, float* weights, int n_tokens,
+                hipStream_t stream);
 // act[t, e * ff + j] = weight(t, e) * relu(up[t, e * ff + j])^2 for chosen experts, 0 for the others
 int ra_moe_relu2_scale(const void* up, void* act, int act_dtype, const int* ids, const float* weights, int top,
                        int experts, int ff, int n_tokens, hipStream_t stream);

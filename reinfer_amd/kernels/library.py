@@ -52,7 +52,7 @@ _SIGNATURES = {
     "ra_tanh_cap": [P, I, I, I, F, P],
     "ra_latent_prep": [P, I, I, I, I, P, I, F, P, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
     "ra_head_linear": [P, I, I, P, P, I, I, P, I, I, I, I, I, I, P],
-    "ra_moe_route": [P, I, I, P, I, I, I, P, P, I, P],
+    "ra_moe_topk": [P, I, I, I, P, P, I, P],
     "ra_moe_relu2_scale": [P, P, I, P, P, I, I, I, I, P],
     "ra_stream_read": [P, c_long, P, P],
     "ra_mfma_loop": [I, I, I, P, P, P],

@@ -263,6 +263,18 @@ class HipKernels:
         if side is not None:
             torch.cuda.current_stream().wait_stream(side)
 
+    def shared_head_limit(self, head_dim: int, block_size: int = 16) -> int:
+        """Query heads that may share one KV head in a call of :meth:`attention` and still take the
+        matrix-core kernels (the decode kernel's waves add their results through LDS, which bounds heads times
+        head size); 0: no number of heads does at this head size. A mixer all of whose heads read one cached
+        row (a shared latent) splits its heads into groups of at most this many."""
+        lib = library.load()
+        for g in range(16, 0, -1):
+            if lib.ra_attention_decode_supports(g, 1, int(head_dim), int(block_size)) \
+                    and lib.ra_attention_prefill_supports(g, 1, int(head_dim), int(block_size)):
+                return g
+        return 0
+
     def _side_stream(self, device):
         s = self._side_streams.get(device)
         if s is None:
@@ -450,8 +462,9 @@ class HipKernels:
         _dev(q, out, kcache, vcache)
         T = batch.num_tokens
         tables = batch.block_tables[group]
-        if out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
-            raise ValueError(f"attention: out {tuple(out.shape)}, expected [{T}, {num_heads * head_dim}]")
+        if out.shape != (T, num_heads * head_dim) or out.stride(1) != 1 or out.dtype != q.dtype:
+            raise ValueError(f"attention: out {tuple(out.shape)}, expected [{T}, {num_heads * head_dim}] with "
+                             "contiguous rows (it may be a column range of a wider buffer)")
         if q.shape[0] != T or q_stride < num_heads * head_dim or q.stride(0) != q_stride:
             raise ValueError("attention: query rows do not match the step's tokens")
         if kcache.dtype != q.dtype or vcache.dtype != q.dtype:
@@ -930,14 +943,15 @@ class HipKernels:
 
     def head_linear(self, x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, o_head: int,
                     gate: Optional[torch.Tensor] = None) -> None:
-        """Products head by head: out[t, h * o_head + n] = sum_k x[t, h * x_head + k] * weight[h, k, n], times
+        """Products head by head: out[t, h * o_head + n] = sum_k x[t, h * x_head + k] * weight[h, n, k], times
         sigmoid(gate[t, h * N + n]) where a gate is given. ``x``, ``out`` and ``gate`` are 2-D with unit
-        column stride (they may be column ranges of wider buffers); ``weight`` is [heads, K, N] contiguous."""
+        column stride (they may be column ranges of wider buffers); ``weight`` is [heads, N, K] contiguous.
+        bfloat16 with K and the strides of ``x`` in steps of 8: matrix cores; else a plain kernel."""
         _dev(x, weight, out, gate)
-        H, K, N = weight.shape
+        H, N, K = weight.shape
         T = x.shape[0]
         if not weight.is_contiguous() or x.dtype != weight.dtype or out.dtype != weight.dtype:
-            raise ValueError("head_linear: weight [heads, K, N] contiguous, all in one dtype")
+            raise ValueError("head_linear: weight [heads, N, K] contiguous, all in one dtype")
         for t, what in ((x, "x"), (out, "out"), (gate, "gate")):
             if t is not None and (t.dim() != 2 or t.shape[0] != T or t.stride(1) != 1 or t.dtype != weight.dtype):
                 raise ValueError(f"head_linear: {what} must be [T, *] rows of the weight's dtype with unit column stride")
@@ -952,20 +966,23 @@ class HipKernels:
     # ---------------------------------------------------- mixture of experts
     def moe_route(self, x: torch.Tensor, router: torch.Tensor, top: int, ids: torch.Tensor,
                   weights: torch.Tensor) -> None:
-        """Float router logits x . router^T, the ``top`` largest a token in falling order into ``ids`` [T, top]
-        (int32) and the softmax over those alone into ``weights`` [T, top] (float32)."""
+        """Router logits x . router^T accumulated and kept in float (``router`` [experts, width] in the
+        activations' dtype: a bfloat16 product's terms are exact in float), the ``top`` largest a token in
+        falling order into ``ids`` [T, top] (int32), the softmax over those alone into ``weights`` [T, top]
+        (float32)."""
         _dev(x, router, ids, weights)
         T, width = x.shape
         E = router.shape[0]
-        if router.shape != (E, width) or router.dtype != torch.float32 or not router.is_contiguous():
-            raise ValueError(f"moe_route: router {tuple(router.shape)} {router.dtype}, expected float32 [experts, {width}]")
-        if x.stride(1) != 1:
-            raise ValueError("moe_route: rows must be contiguous")
+        if router.shape != (E, width) or router.dtype != x.dtype or not router.is_contiguous():
+            raise ValueError(f"moe_route: router {tuple(router.shape)} {router.dtype}, expected [experts, {width}] "
+                             "in the activations' dtype")
         if ids.shape != (T, top) or ids.dtype != torch.int32 or not ids.is_contiguous() \
                 or weights.shape != (T, top) or weights.dtype != torch.float32 or not weights.is_contiguous():
             raise ValueError(f"moe_route: ids int32 and weights float32, both [{T}, {top}]")
-        library.call("ra_moe_route", x.data_ptr(), _tag(x, "moe_route"), x.stride(0), router.data_ptr(), E, width,
-                     int(top), ids.data_ptr(), weights.data_ptr(), T, _stream())
+        logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
+        self.linear(x, router, logits)
+        library.call("ra_moe_topk", logits.data_ptr(), logits.stride(0), E, int(top), ids.data_ptr(),
+                     weights.data_ptr(), T, _stream())
 
     def moe_relu2_scale(self, up: torch.Tensor, act: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
                         experts: int, ff: int) -> None:

@@ -80,10 +80,10 @@ class LatentAttention:
         self.proj_width += pad
         self.w_in = torch.cat(rows, dim=0).contiguous()
         self.c_norm = weights[prefix + "dkv.norm"]
-        # head products, [heads, K, N] with N contiguous: queries through the key matrices, W_uk[a, d, r] as stored;
-        # results through the value matrices, W_uv[a, v, r] transposed to [a, r, v]
-        self.w_absorb = weights[prefix + "uk"].view(H, D, self.rank).contiguous()
-        self.w_values = weights[prefix + "uv"].view(H, Dv, self.rank).transpose(1, 2).contiguous()
+        # head products, [heads, N, K] with K contiguous: queries through the key matrices, W_uk[a, d, r] transposed
+        # to [a, r, d]; results through the value matrices, W_uv[a, v, r] as stored
+        self.w_absorb = weights[prefix + "uk"].view(H, D, self.rank).transpose(1, 2).contiguous()
+        self.w_values = weights[prefix + "uv"].view(H, Dv, self.rank).contiguous()
         self.w_o = weights[prefix + "o"]
         self.position = lookup("position", spec.position.kind)(spec.position, device)
         if self.position.rotary_dim > R:
@@ -96,6 +96,29 @@ class LatentAttention:
         hook = getattr(kernels.current(), "plan_captured_step", None)
         if hook is not None:
             hook(batch, num_rows, ctx_cap)
+
+    def _head_groups(self, ops, cache: LayerCache):
+        """(first head, heads) of each attention call: all heads at once where the kernels take that many
+        query heads on one KV head, else even groups of as many as they take."""
+        H = self.num_heads
+        groups = getattr(self, "_groups", None)
+        if groups is None:
+            limit = 0
+            ask = getattr(ops, "shared_head_limit", None)
+            if ask is not None and self.dtype == torch.bfloat16:
+                limit = int(ask(self.cache_dim, cache.k.shape[2] * 16))
+            if limit <= 0 or H <= limit:
+                groups = [(0, H)]
+            else:
+                n = -(-H // limit)
+                base, extra = divmod(H, n)
+                groups, a = [], 0
+                for i in range(n):
+                    g = base + (1 if i < extra else 0)
+                    groups.append((a, g))
+                    a += g
+            self._groups = groups
+        return groups
 
     def forward(self, x, batch, cache: LayerCache, resid: Optional[torch.Tensor] = None):
         ops = kernels.current()
@@ -114,8 +137,10 @@ class LatentAttention:
         else:
             q_lat[:, :, :self.rank].zero_()
         o_lat = torch.empty((T, H * Dp), dtype=self.dtype, device=x.device)
-        ops.attention(q_rows, H * Dp, o_lat, cache.k, cache.v, batch, H, 1, Dp, self.scale, self.window,
-                      cache.group)
+        for a, g in self._head_groups(ops, cache):
+            # heads a .. a + g - 1 against the one cached row a token: column ranges of the same buffers
+            ops.attention(q_rows[:, a * Dp:], H * Dp, o_lat[:, a * Dp:(a + g) * Dp], cache.k, cache.v, batch, g, 1,
+                          Dp, self.scale, self.window, cache.group)
         heads = torch.empty((T, H * Dv), dtype=self.dtype, device=x.device)
         ops.head_linear(o_lat, Dp, self.w_values, heads, Dv,
                         gate=proj[:, self.gate_off:self.gate_off + H * Dv] if self.gated else None)

@@ -49,7 +49,7 @@ class MixtureOfExperts:
         self.experts, self.top, self.ff = int(p.experts), int(p.top), int(spec.intermediate)
         self.w_up = torch.cat([weights[f"{prefix}e{e}.up"] for e in range(self.experts)], dim=0).contiguous()
         self.w_down = torch.cat([weights[f"{prefix}e{e}.down"] for e in range(self.experts)], dim=1).contiguous()
-        self.router = weights[prefix + "router"].to(torch.float32).contiguous()      # logits are float
+        self.router = weights[prefix + "router"]            # logits are accumulated and kept in float
 
     def forward(self, x, batch, resid: Optional[torch.Tensor] = None):
         ops = kernels.current()

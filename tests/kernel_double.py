@@ -153,9 +153,9 @@ class KernelDouble:
             vflat[s // bs][:, v_index(s % bs, e, Dp)] = row[t].to(vcache.dtype)
 
     def head_linear(self, x, x_head, weight, out, o_head, gate=None):
-        H, K, N = weight.shape
+        H, N, K = weight.shape
         for h in range(H):
-            y = x[:, h * x_head:h * x_head + K].float() @ weight[h].float()
+            y = x[:, h * x_head:h * x_head + K].float() @ weight[h].float().T
             if gate is not None:
                 y = y * torch.sigmoid(gate[:, h * N:(h + 1) * N].float())
             out[:, h * o_head:h * o_head + N] = y.to(out.dtype)

@@ -1,7 +1,7 @@
 """Tiny Puresun configurations and model folders for the tests.
 
 The configurations differ in every size and option: layer count and order, width (a multiple of 8 or not),
-heads (1, 2, 3, 5, 20: more than the 16 the decode kernel's groups take), unrotated / rotated / value sizes,
+heads (1, 2, 3, 18, 20: more than the 16 that share a KV head in the matrix-core kernels), unrotated / rotated / value sizes,
 latent ranks whose cache row is a multiple of 16 or needs padding, windows (4 to 40, none), rotation base,
 experts and how many are chosen (all of them, some, one of one), layers without a feed-forward, the
 repeated run (at the start, in the middle, once, three times, none), the token-pair table, the logit cap.
@@ -57,7 +57,7 @@ PS_B = {
     "architecture": "Puresun", "vocab": 257, "width": 64, "norm": {"eps": 1e-5},
     "layers": [
         _layer(_mixer(1, 32, 16, 32, 64, 4), _moe(4, 4, 16)),
-        _layer(_mixer(5, 16, 16, 8, 48, 40, base=1000000.0), _moe(1, 1, 72)),
+        _layer(_mixer(18, 16, 16, 8, 48, 40, base=1000000.0), _moe(1, 1, 72)),
     ],
 }
 # a width that is no multiple of 8, 20 heads, a cache row of 106 -> 112, no window on the second layer,

@@ -127,20 +127,24 @@ def test_latent_prep(dtype, H, D, R, rot, rank):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,H,K,N", [(1, 3, 16, 40), (17, 2, 24, 8), (70, 5, 100, 4), (33, 1, 96, 300)])
-def test_head_linear(dtype, T, H, K, N):
+@pytest.mark.parametrize("T,H,K,N,pad", [(1, 3, 16, 40, 7), (17, 2, 24, 8, 8), (70, 5, 100, 4, 7), (33, 1, 96, 300, 0),
+                                         (16, 3, 40, 24, 8), (130, 2, 64, 50, 16), (5, 18, 128, 192, 64)])
+def test_head_linear(dtype, T, H, K, N, pad):
+    """Odd sizes and strides (the plain kernel) and sizes in steps of 8 (matrix cores in bfloat16): token
+    counts on both sides of the tiles of 16 and 64, column counts that end inside a tile."""
     g = torch.Generator().manual_seed(4)
-    x_head, o_head = K + 7, N + 3
-    x = torch.randn(T, 5 + H * x_head, generator=g).to(dtype).to(DEV)
-    w = (torch.randn(H, K, N, generator=g) / math.sqrt(K)).to(dtype).to(DEV)
+    x_head, o_head = K + pad, N + 3
+    lead = 5 if pad == 7 else 8
+    x = torch.randn(T, lead + H * x_head, generator=g).to(dtype).to(DEV)
+    w = (torch.randn(H, N, K, generator=g) / math.sqrt(K)).to(dtype).to(DEV)
     gate = torch.randn(T, H * N + 2, generator=g).to(dtype).to(DEV)
     for use_gate in (False, True):
         out = torch.full((T, H * o_head), float("nan"), dtype=dtype, device=DEV)
-        ops().head_linear(x[:, 5:], x_head, w, out, o_head, gate=gate if use_gate else None)
+        ops().head_linear(x[:, lead:], x_head, w, out, o_head, gate=gate if use_gate else None)
         got = out.float().cpu().view(T, H, o_head)
         assert torch.isnan(got[:, :, N:]).all()
-        xs = x.float().cpu()[:, 5:].view(T, H, x_head)[:, :, :K]
-        want = torch.einsum("thk,hkn->thn", xs, w.float().cpu())
+        xs = x.float().cpu()[:, lead:].view(T, H, x_head)[:, :, :K]
+        want = torch.einsum("thk,hnk->thn", xs, w.float().cpu())
         if use_gate:
             want = want * torch.sigmoid(gate.float().cpu()[:, :H * N].view(T, H, N))
         close(got[:, :, :N], want, dtype)
@@ -152,11 +156,11 @@ def test_moe_route(dtype, E, top, width):
     g = torch.Generator().manual_seed(5)
     T = 19
     x = torch.randn(T, width + 8, generator=g).to(dtype).to(DEV)[:, :width]
-    router = torch.randn(E, width, generator=g).to(DEV)
+    router = torch.randn(E, width, generator=g).to(dtype).to(DEV)
     ids = torch.full((T, top), -1, dtype=torch.int32, device=DEV)
     wts = torch.full((T, top), float("nan"), dtype=torch.float32, device=DEV)
     ops().moe_route(x, router, top, ids, wts)
-    z = x.float().cpu().double() @ router.cpu().double().T
+    z = x.float().cpu().double() @ router.float().cpu().double().T
     val, idx = torch.topk(z, top, dim=-1)
     assert ids.cpu().tolist() == idx.tolist()
     close(wts, torch.softmax(val, dim=-1), torch.float32)
@@ -168,9 +172,10 @@ def test_moe_route(dtype, E, top, width):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_moe_relu2_scale(dtype):
+@pytest.mark.parametrize("ff", [20, 24])
+def test_moe_relu2_scale(dtype, ff):
     g = torch.Generator().manual_seed(6)
-    T, E, ff, top = 11, 6, 20, 3
+    T, E, top = 11, 6, 3
     up = torch.randn(T, E * ff, generator=g).to(dtype).to(DEV)
     ids = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).to(torch.int32).to(DEV)
     wts = torch.rand(T, top, generator=g).to(DEV)
