@@ -36,10 +36,10 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
   for (int i = lane; i < d; i += RA_WAVE) qs[i] = to_f32(qv[i]);
   __syncthreads();
 
-  const int n_acc = (d + RA_WAVE - 1) / RA_WAVE;   // output elements per lane (<= 8)
-  float acc[8];
+  const int n_acc = (d + RA_WAVE - 1) / RA_WAVE;   // output elements per lane (<= 16)
+  float acc[16];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
   float m = -INFINITY, l = 0.f;
 
   for (int base = lo; base <= p; base += RA_WAVE) {
@@ -64,7 +64,7 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
     __syncthreads();
     const int n_keys = (p - base + 1 < RA_WAVE) ? p - base + 1 : RA_WAVE;
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
+    for (int r = 0; r < 16; ++r) {
       if (r < n_acc) {
         const int i = r * RA_WAVE + lane;
         float sum = 0.f;
@@ -83,7 +83,7 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
   TA* o = out + (size_t)t * out_stride + (size_t)a * d;
   const float inv = 1.f / l;
 #pragma unroll
-  for (int r = 0; r < 8; ++r) {
+  for (int r = 0; r < 16; ++r) {
     if (r < n_acc) {
       const int i = r * RA_WAVE + lane;
       if (i < d) o[i] = from_f32<TA>(acc[r] * inv);
@@ -98,7 +98,7 @@ extern "C" int ra_attention_plain(const void* q, int q_stride, void* out, int ou
                                   int d, float scale, int window, hipStream_t stream) {
   RA_CHECK(n_tokens > 0, "attention_plain: no tokens");
   RA_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "attention_plain: %d query heads do not divide into %d groups", Hq, Hkv);
-  RA_CHECK(d > 0 && d <= 512, "attention_plain: head size %d outside 1..512", d);
+  RA_CHECK(d > 0 && d <= 1024, "attention_plain: head size %d outside 1..1024", d);
   RA_CHECK(block_size > 0 && block_size % 16 == 0 && d % 16 == 0 && max_blocks > 0,
            "attention_plain: the cache is tiled 16 x 16: block size %d and head size %d must be multiples of 16",
            block_size, d);

@@ -76,7 +76,15 @@ PS_C = {
 PS_A16 = json.loads(json.dumps(PS_A))
 PS_A16["layers"][0]["mlp"] = _moe(4, 4, 24)
 
-CONFIGS = {"A": (PS_A, 11), "B": (PS_B, 12), "C": (PS_C, 13), "A16": (PS_A16, 14)}
+# a latent wider than the matrix-core attention kernels' largest head (288 > 256): the plain kernel in both dtypes
+PS_D = {
+    "architecture": "Puresun", "vocab": 90, "width": 32, "norm": {"eps": 1e-6},
+    "embedding": {"bigram": {"buckets": 10, "mul_prev": 1, "mul_cur": 1}},
+    "layers": [_layer(_mixer(2, 8, 8, 8, 280, 12), _moe(2, 2, 8))],
+    "loop": {"start": 0, "stop": 1, "times": 1},
+}
+
+CONFIGS = {"A": (PS_A, 11), "B": (PS_B, 12), "C": (PS_C, 13), "A16": (PS_A16, 14), "D": (PS_D, 15)}
 
 # deviation of the random matrices by the last part of their name (norm weights are uniform on [0.8, 1.2))
 STD = {"embed": 1.0, "bigram": 0.5, "loop.step": 0.5, "router": 0.6, "head": 0.3, "default": 0.15}

@@ -161,7 +161,7 @@ CHECKS = [check_whole_and_one_by_one, check_portions, check_mixed_with_reuse, ch
 
 # ------------------------------------------------------------------ CPU: bookkeeping on the stand-in
 @pytest.mark.parametrize("check", CHECKS, ids=lambda f: f.__name__)
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_engine_bookkeeping_cpu(tmp_path_factory, check, which):
     folder = make_folder(tmp_path_factory.getbasetemp(), which, "float32")
     with kernels.use(KernelDouble()):
@@ -188,7 +188,8 @@ def test_previous_token_is_request_state_cpu(tmp_path_factory):
 
 
 # ------------------------------------------------------------------ GPU: the real kernels
-GPU_CASES = [("A", "float32"), ("B", "float32"), ("C", "float32"), ("A16", "bfloat16"), ("B", "bfloat16")]
+GPU_CASES = [("A", "float32"), ("B", "float32"), ("C", "float32"), ("A16", "bfloat16"), ("B", "bfloat16"),
+             ("D", "float32"), ("D", "bfloat16")]
 
 
 @pytest.mark.gpu
