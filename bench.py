@@ -442,16 +442,18 @@ def design_run(args) -> int:
             rec = {}
             ms = prefill_run(engine, fake, 2048, 3, args.seed + 1)
             rec["prefill_2048_tok_s"] = round(2048 / (ms * 1e-3), 1)
-            for b in (8, 64):
+            for b in (1, 8, 64):
                 dms, ctx = decode_run(engine, fake, b, 1536, 32, 8, args.seed + 2 + b, b + 32 + 8 + 16)
                 rec[f"decode_b{b}_tok_s"] = round(b / (dms * 1e-3), 1)
                 rec[f"decode_b{b}_ms"] = round(dms, 3)
             rec["prefill_2048_classes"] = classes(engine, vocab, 2048, 1, 0)
             rec["decode_b8_classes"] = classes(engine, vocab, 1, 8, 1536)
-            log(f"{name} {which}: prefill {rec['prefill_2048_tok_s']:.0f} tok/s, decode batch 8 "
+            rec["decode_b1_classes"] = classes(engine, vocab, 1, 1, 1536)
+            log(f"{name} {which}: prefill {rec['prefill_2048_tok_s']:.0f} tok/s, decode batch 1 "
+                f"{rec['decode_b1_tok_s']:.0f} tok/s ({rec['decode_b1_ms']} ms), batch 8 "
                 f"{rec['decode_b8_tok_s']:.0f} tok/s ({rec['decode_b8_ms']} ms), batch 64 {rec['decode_b64_tok_s']:.0f} tok/s "
                 f"({rec['decode_b64_ms']} ms)")
-            for step in ("prefill_2048_classes", "decode_b8_classes"):
+            for step in ("prefill_2048_classes", "decode_b8_classes", "decode_b1_classes"):
                 for label, row in rec[step].items():
                     log(f"    {step[:-8]:13s} {label:40s} {row['ms']:8.3f} ms  {row['calls']:4d} calls  of roofline {row['of_roofline']}")
             results.setdefault(name, {})[which] = rec

@@ -133,3 +133,139 @@ extern "C" int ra_moe_relu2_scale(const void* up, void* act, int act_dtype, cons
   RA_LAUNCH_CHECK("moe_relu2_scale");
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Few tokens (a decode step of one or two requests): only the chosen experts' rows are read. Pair p = (token
+// t, choice j) with expert e = ids[p] and weight g = weights[p]:
+//   act[p, f]   = g * relu(W_up[e * ff + f, :] . x[t, :])^2          one wave a row f, lanes split the width
+//   y[t, n]     = sum_j W_down[n, e_j * ff : (e_j + 1) * ff] . act[p_j, :]   one wave a column n, added into the
+//                 float stream (resid) or written to out
+// bfloat16 rows in steps of 8 are read 16 bytes a lane; anything else element by element. Sums are float.
+// ---------------------------------------------------------------------------
+// s[r] += w_r . v for four rows w_0..w_3 that share v: the lanes split K; rows of bfloat16 in steps of 8 are
+// read 16 bytes a lane, four loads in flight beside the shared one
+template <typename TA>
+__device__ __forceinline__ void moe_dot4(const TA* const (&w)[4], const TA* __restrict__ v, int K, int lane, bool vec,
+                                         float (&s)[4]) {
+  for (int k = lane; k < K; k += RA_WAVE) {
+    const float b = to_f32(v[k]);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s[r] += to_f32(w[r][k]) * b;
+  }
+}
+template <>
+__device__ __forceinline__ void moe_dot4<bf16_t>(const bf16_t* const (&w)[4], const bf16_t* __restrict__ v, int K,
+                                                 int lane, bool vec, float (&s)[4]) {
+  if (vec) {
+    for (int k = lane * 8; k < K; k += RA_WAVE * 8) {
+      const bf16x8_t b = *(const bf16x8_t*)(v + k);
+      bf16x8_t a[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) a[r] = *(const bf16x8_t*)(w[r] + k);
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s[r] += (float)a[r][i] * (float)b[i];
+    }
+  } else {
+    for (int k = lane; k < K; k += RA_WAVE) {
+      const float b = (float)v[k];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[r] += (float)w[r][k] * b;
+    }
+  }
+}
+
+#define MOE_ROWS 16          // rows (or columns) a workgroup of four waves takes, four a wave
+template <typename TA>
+__global__ void __launch_bounds__(256)
+moe_up_chosen_kernel(const TA* __restrict__ x, int ldx, const TA* __restrict__ Wup, const int* __restrict__ ids,
+                     const float* __restrict__ weights, TA* __restrict__ act, int ff, int width, int top, int vec) {
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE;
+  const int p = blockIdx.y;
+  const int t = p / top;
+  const int e = ids[p];
+  const float g = weights[p];
+  const int f0 = blockIdx.x * MOE_ROWS + wave * 4;
+  if (f0 >= ff) return;
+  const TA* w[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) w[r] = Wup + ((size_t)e * ff + (f0 + r < ff ? f0 + r : f0)) * width;   // past the end: a row again, not stored
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  moe_dot4<TA>(w, x + (size_t)t * ldx, width, lane, vec != 0, s);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) s[r] = wave_sum(s[r]);
+  if (lane < 4 && f0 + lane < ff) {
+    const float u = fmaxf(lane == 0 ? s[0] : lane == 1 ? s[1] : lane == 2 ? s[2] : s[3], 0.f);
+    act[(size_t)p * ff + f0 + lane] = from_f32<TA>(g * (u * u));
+  }
+}
+
+template <typename TA>
+__global__ void __launch_bounds__(256)
+moe_down_chosen_kernel(const TA* __restrict__ act, const TA* __restrict__ Wdown, const int* __restrict__ ids,
+                       float* __restrict__ resid, TA* __restrict__ out, int ff, int width, int E, int top, int vec) {
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE;
+  const int t = blockIdx.y;
+  const int n0 = blockIdx.x * MOE_ROWS + wave * 4;
+  if (n0 >= width) return;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < top; ++j) {               // choice order: the same sum whatever else is in the step
+    const int p = t * top + j;
+    const TA* w[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) w[r] = Wdown + (size_t)(n0 + r < width ? n0 + r : n0) * E * ff + (size_t)ids[p] * ff;
+    moe_dot4<TA>(w, act + (size_t)p * ff, ff, lane, vec != 0, s);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) s[r] = wave_sum(s[r]);
+  if (lane < 4 && n0 + lane < width) {
+    const float v = lane == 0 ? s[0] : lane == 1 ? s[1] : lane == 2 ? s[2] : s[3];
+    const size_t at = (size_t)t * width + n0 + lane;
+    if (resid) resid[at] += v;                   // this thread alone owns (t, n)
+    else out[at] = from_f32<TA>(v);
+  }
+}
+
+extern "C" int ra_moe_up_chosen(const void* x, int ldx, const void* w_up, const int* ids, const float* weights,
+                                void* act, int act_dtype, int n_tokens, int top, int experts, int ff, int width,
+                                hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && top > 0 && top <= experts && ff > 0 && width > 0 && ldx >= width,
+           "moe_up_chosen: %d tokens, %d of %d experts of %d x %d", n_tokens, top, experts, ff, width);
+  RA_CHECK((long)n_tokens * top <= 65535, "moe_up_chosen: %d pairs in one launch", n_tokens * top);
+  const int vec = (width % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w_up % 16) == 0) ? 1 : 0;
+  dim3 grid((ff + MOE_ROWS - 1) / MOE_ROWS, n_tokens * top);
+  if (act_dtype == RA_F32)
+    moe_up_chosen_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, ldx, (const float*)w_up, ids, weights,
+                                                          (float*)act, ff, width, top, 0);
+  else if (act_dtype == RA_BF16)
+    moe_up_chosen_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w_up, ids, weights,
+                                                           (bf16_t*)act, ff, width, top, vec);
+  else
+    return ra_fail("moe_up_chosen: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("moe_up_chosen");
+  return 0;
+}
+
+extern "C" int ra_moe_down_chosen(const void* act, const void* w_down, const int* ids, float* resid, void* out,
+                                  int act_dtype, int n_tokens, int top, int experts, int ff, int width,
+                                  hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && top > 0 && top <= experts && ff > 0 && width > 0,
+           "moe_down_chosen: %d tokens, %d of %d experts of %d x %d", n_tokens, top, experts, ff, width);
+  RA_CHECK((resid != nullptr) != (out != nullptr), "moe_down_chosen: the result goes into the stream or into out");
+  RA_CHECK(n_tokens <= 65535, "moe_down_chosen: %d tokens in one launch", n_tokens);
+  const int vec = (ff % 8 == 0 && ((uintptr_t)act % 16) == 0 && ((uintptr_t)w_down % 16) == 0) ? 1 : 0;
+  dim3 grid((width + MOE_ROWS - 1) / MOE_ROWS, n_tokens);
+  if (act_dtype == RA_F32)
+    moe_down_chosen_kernel<float><<<grid, 256, 0, stream>>>((const float*)act, (const float*)w_down, ids, resid,
+                                                            (float*)out, ff, width, experts, top, 0);
+  else if (act_dtype == RA_BF16)
+    moe_down_chosen_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)w_down, ids, resid,
+                                                             (bf16_t*)out, ff, width, experts, top, vec);
+  else
+    return ra_fail("moe_down_chosen: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("moe_down_chosen");
+  return 0;
+}

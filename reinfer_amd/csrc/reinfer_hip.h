@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 18
+#define RA_ABI_VERSION 19
 
 #ifdef __cplusplus
 extern "C" {
@@ -200,6 +200,15 @@ int ra_moe_topk(const float* logits, int ld, int experts, int top, int* ids, flo
 // act[t, e * ff + j] = weight(t, e) * relu(up[t, e * ff + j])^2 for chosen experts, 0 for the others
 int ra_moe_relu2_scale(const void* up, void* act, int act_dtype, const int* ids, const float* weights, int top,
                        int experts, int ff, int n_tokens, hipStream_t stream);
+
+// Few tokens: only the chosen experts' rows are read. w_up [experts * ff, width], w_down [width, experts * ff];
+// act[t * top + j, f] = weights[t, j] * relu(w_up[ids[t, j] * ff + f, :] . x[t, :])^2, then
+// y[t, n] = sum_j w_down[n, ids[t, j] * ff : ...] . act[t * top + j, :], added into resid (float [n_tokens, width])
+// or written to out ([n_tokens, width], the activations' dtype): exactly one of the two is given
+int ra_moe_up_chosen(const void* x, int ldx, const void* w_up, const int* ids, const float* weights, void* act,
+                     int act_dtype, int n_tokens, int top, int experts, int ff, int width, hipStream_t stream);
+int ra_moe_down_chosen(const void* act, const void* w_down, const int* ids, float* resid, void* out, int act_dtype,
+                       int n_tokens, int top, int experts, int ff, int width, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 
 class KernelLibraryError(RuntimeError):
@@ -54,6 +54,8 @@ _SIGNATURES = {
     "ra_head_linear": [P, I, I, P, P, I, I, P, I, I, I, I, I, I, P],
     "ra_moe_topk": [P, I, I, I, P, P, I, P],
     "ra_moe_relu2_scale": [P, P, I, P, P, I, I, I, I, P],
+    "ra_moe_up_chosen": [P, I, P, P, P, P, I, I, I, I, I, I, P],
+    "ra_moe_down_chosen": [P, P, P, P, P, I, I, I, I, I, I, P],
     "ra_stream_read": [P, c_long, P, P],
     "ra_mfma_loop": [I, I, I, P, P, P],
 }

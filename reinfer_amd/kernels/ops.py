@@ -999,6 +999,60 @@ class HipKernels:
         library.call("ra_moe_relu2_scale", up.data_ptr(), act.data_ptr(), _tag(up, "moe_relu2_scale"), ids.data_ptr(),
                      weights.data_ptr(), top, int(experts), int(ff), T, _stream())
 
+    # Steps of so few tokens that their choices name at most this share of the experts read only the chosen
+    # experts' rows (two kernels, a wave a row) instead of running every expert through the matrix cores
+    MOE_CHOSEN_SHARE = 0.5
+    MOE_CHOSEN_TOKENS = 8
+
+    def moe_reads_chosen(self, n_tokens: int, top: int, experts: int) -> bool:
+        """Whether a step of ``n_tokens`` should read only its chosen experts (``moe_up_chosen`` /
+        ``moe_down_chosen``): its token-expert pairs are few against the experts there are."""
+        return n_tokens <= self.MOE_CHOSEN_TOKENS and n_tokens * top <= self.MOE_CHOSEN_SHARE * experts
+
+    def moe_up_chosen(self, x: torch.Tensor, w_up: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+                      act: torch.Tensor, ff: int) -> None:
+        """act[t * top + j] = weights[t, j] * relu(w_up[ids[t, j] * ff : ... + ff] . x[t])^2 for the chosen
+        experts only; ``w_up`` is [experts * ff, width], ``act`` [T * top, ff]."""
+        _dev(x, w_up, ids, weights, act)
+        T, width = x.shape
+        top = ids.shape[1]
+        E = w_up.shape[0] // ff
+        if w_up.shape != (E * ff, width) or not w_up.is_contiguous() or x.dtype != w_up.dtype or x.stride(1) != 1:
+            raise ValueError(f"moe_up_chosen: x {tuple(x.shape)}, w_up {tuple(w_up.shape)} for experts of {ff}")
+        if act.shape != (T * top, ff) or act.dtype != x.dtype or not act.is_contiguous():
+            raise ValueError(f"moe_up_chosen: act {tuple(act.shape)}, expected [{T * top}, {ff}]")
+        self._check_choice("moe_up_chosen", ids, weights, T, top)
+        library.call("ra_moe_up_chosen", x.data_ptr(), x.stride(0), w_up.data_ptr(), ids.data_ptr(),
+                     weights.data_ptr(), act.data_ptr(), _tag(x, "moe_up_chosen"), T, top, E, int(ff), width, _stream())
+
+    def moe_down_chosen(self, act: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, ff: int,
+                        resid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> None:
+        """y[t] = sum_j w_down[:, ids[t, j] * ff : ... + ff] . act[t * top + j], added into the float ``resid``
+        or written to ``out`` (exactly one is given); ``w_down`` is [width, experts * ff]."""
+        _dev(act, w_down, ids, resid, out)
+        T, top = ids.shape
+        width = w_down.shape[0]
+        E = w_down.shape[1] // ff
+        if w_down.shape != (width, E * ff) or not w_down.is_contiguous() or act.dtype != w_down.dtype \
+                or act.shape != (T * top, ff) or not act.is_contiguous():
+            raise ValueError(f"moe_down_chosen: act {tuple(act.shape)}, w_down {tuple(w_down.shape)} for experts of {ff}")
+        if ids.dtype != torch.int32 or not ids.is_contiguous():
+            raise ValueError("moe_down_chosen: ids are contiguous int32 [T, top]")
+        if (resid is None) == (out is None):
+            raise ValueError("moe_down_chosen: the result goes into the stream or into out")
+        if resid is not None and (resid.shape != (T, width) or resid.dtype != torch.float32 or not resid.is_contiguous()):
+            raise ValueError("moe_down_chosen: the residual stream is contiguous float32 [T, width]")
+        if out is not None and (out.shape != (T, width) or out.dtype != act.dtype or not out.is_contiguous()):
+            raise ValueError("moe_down_chosen: out is contiguous [T, width] in the activations' dtype")
+        library.call("ra_moe_down_chosen", act.data_ptr(), w_down.data_ptr(), ids.data_ptr(), _ptr(resid), _ptr(out),
+                     _tag(act, "moe_down_chosen"), T, top, E, int(ff), width, _stream())
+
+    @staticmethod
+    def _check_choice(what: str, ids, weights, T: int, top: int) -> None:
+        if ids.shape != (T, top) or ids.dtype != torch.int32 or not ids.is_contiguous() \
+                or weights.shape != (T, top) or weights.dtype != torch.float32 or not weights.is_contiguous():
+            raise ValueError(f"{what}: ids int32 and weights float32, both [{T}, {top}]")
+
     # -------------------------------------------------------------- sampling
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, seeds: torch.Tensor,
                positions: torch.Tensor, tokens: torch.Tensor) -> None:

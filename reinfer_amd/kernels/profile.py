@@ -30,7 +30,8 @@ _ATTN = {"attention", "attention_plain", "attention_decode", "attention_prefill"
 _LINEAR = {"linear", "linear_plain", "linear_skinny", "gated_linear", "linear_ranges"}
 # kernels of further mechanisms, each a class of its own
 _OTHER = {"latent_prep": "latent norm + rotation + cache write", "head_linear": "products head by head",
-          "moe_route": "router", "moe_relu2_scale": "expert activation", "stream_add": "stream add",
+          "moe_route": "router", "moe_relu2_scale": "expert activation",
+          "moe_up_chosen": "chosen experts up", "moe_down_chosen": "chosen experts down", "stream_add": "stream add",
           "pair_hash_add": "embedding", "tanh_cap": "logit cap"}
 
 
@@ -83,6 +84,8 @@ class TimedKernels:
             if isinstance(w, torch.Tensor) and isinstance(args[0], torch.Tensor):
                 nbytes = w.numel() * w.element_size()
                 flops = 2 * args[0].shape[0] * w.numel()
+            if attr == "linear_ranges" and out is None:
+                return out                # it declined (the caller runs the whole product next): nothing was launched
             self._spans.append((self._label(attr, args, kwargs), e0, e1, nbytes, flops))
             return out
         return timed_call

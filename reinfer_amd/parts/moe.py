@@ -8,7 +8,9 @@ The experts' up projections are laid side by side as one [experts * ff, width] m
 projections as one [width, experts * ff] matrix. A step computes every expert's up projection in one product,
 applies the activation and the routing weight in one kernel (0 for experts a token did not choose), and one
 product with the down matrix is then the weighted sum: with few experts of which a good share is chosen, two
-dense products at the matrix cores' rate cost less than gathering tokens by expert would.
+dense products at the matrix cores' rate cost less than gathering tokens by expert would. A step of so few
+tokens that most experts are not asked for at all (one or two requests decoding) reads only the chosen experts'
+rows instead, a wave a row.
 """
 from __future__ import annotations
 
@@ -58,6 +60,17 @@ class MixtureOfExperts:
         ids = torch.empty((T, self.top), dtype=torch.int32, device=x.device)
         weights = torch.empty((T, self.top), dtype=torch.float32, device=x.device)
         ops.moe_route(x, self.router, self.top, ids, weights)
+        chosen = getattr(ops, "moe_reads_chosen", None)
+        if chosen is not None and chosen(T, self.top, self.experts):
+            # so few tokens that most experts are not asked for: only the chosen experts' rows are read
+            act = torch.empty((T * self.top, self.ff), dtype=self.dtype, device=x.device)
+            ops.moe_up_chosen(x, self.w_up, ids, weights, act, self.ff)
+            if resid is not None:
+                ops.moe_down_chosen(act, self.w_down, ids, self.ff, resid=resid)
+                return None
+            out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
+            ops.moe_down_chosen(act, self.w_down, ids, self.ff, out=out)
+            return out
         up = torch.empty((T, n), dtype=self.dtype, device=x.device)
         ops.linear(x, self.w_up, up)
         act = torch.empty((T, n), dtype=self.dtype, device=x.device)

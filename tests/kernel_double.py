@@ -174,6 +174,27 @@ class KernelDouble:
         u = torch.relu(up.float()).view(T, experts, ff)
         act.copy_((gate[:, :, None] * u * u).view(T, experts * ff).to(act.dtype))
 
+    def moe_reads_chosen(self, n_tokens, top, experts):
+        return n_tokens <= 8 and n_tokens * top <= 0.5 * experts
+
+    def moe_up_chosen(self, x, w_up, ids, weights, act, ff):
+        T, top = ids.shape
+        for t in range(T):
+            for j in range(top):
+                e = int(ids[t, j])
+                u = torch.relu(w_up[e * ff:(e + 1) * ff].float() @ x[t].float())
+                act[t * top + j] = (float(weights[t, j]) * u * u).to(act.dtype)
+
+    def moe_down_chosen(self, act, w_down, ids, ff, resid=None, out=None):
+        T, top = ids.shape
+        for t in range(T):
+            y = sum(w_down[:, int(ids[t, j]) * ff:(int(ids[t, j]) + 1) * ff].float() @ act[t * top + j].float()
+                    for j in range(top))
+            if resid is not None:
+                resid[t] += y
+            else:
+                out[t] = y.to(out.dtype)
+
     GATE_GROUP = 8
 
     def silu_mul(self, gate_up, out, group=0):

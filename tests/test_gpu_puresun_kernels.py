@@ -186,3 +186,31 @@ def test_moe_relu2_scale(dtype, ff):
     u = torch.relu(up.float().cpu()).view(T, E, ff)
     close(act, (gate[:, :, None] * u * u).view(T, E * ff), dtype)
     assert (act.float().cpu().view(T, E, ff)[gate == 0] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,E,top,ff,width", [(1, 6, 2, 24, 48), (2, 9, 3, 20, 36), (3, 16, 1, 64, 128), (1, 5, 5, 8, 200)])
+def test_moe_chosen_experts(dtype, T, E, top, ff, width):
+    """Only the chosen experts' rows: against all experts computed plainly and weighted, into the stream and
+    into a result of its own; sizes in steps of 8 (16-byte reads) and not."""
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(T, width, generator=g).to(dtype).to(DEV)
+    w_up = (torch.randn(E * ff, width, generator=g) / math.sqrt(width)).to(dtype).to(DEV)
+    w_down = (torch.randn(width, E * ff, generator=g) / math.sqrt(ff)).to(dtype).to(DEV)
+    ids = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).to(torch.int32).to(DEV)
+    wts = torch.rand(T, top, generator=g).to(DEV)
+    act = torch.full((T * top, ff), float("nan"), dtype=dtype, device=DEV)
+    ops().moe_up_chosen(x, w_up, ids, wts, act, ff)
+    xf, uf, df = x.float().cpu(), w_up.float().cpu().view(E, ff, width), w_down.float().cpu().view(width, E, ff)
+    want_act = torch.stack([float(wts[t, j]) * torch.relu(uf[int(ids[t, j])] @ xf[t]) ** 2
+                            for t in range(T) for j in range(top)])
+    close(act, want_act, dtype)
+    a = act.float().cpu().view(T, top, ff)
+    want = torch.stack([sum(df[:, int(ids[t, j])] @ a[t, j] for j in range(top)) for t in range(T)])
+    out = torch.full((T, width), float("nan"), dtype=dtype, device=DEV)
+    ops().moe_down_chosen(act, w_down, ids, ff, out=out)
+    close(out, want, dtype)
+    resid = torch.randn(T, width, generator=g).to(DEV)
+    base = resid.clone().cpu()
+    ops().moe_down_chosen(act, w_down, ids, ff, resid=resid)
+    close(resid, base + want, torch.float32 if dtype == torch.float32 else dtype)

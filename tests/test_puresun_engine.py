@@ -269,3 +269,35 @@ def test_captured_decode_steps_gpu(tmp_path_factory):
     for r, toks in seqs.items():
         assert rel_err(outs[0][r], outs[1][r]) < 1e-6, r
         assert rel_err(outs[0][r], reference(folder, toks)) < TOL["float32"], r
+
+
+def test_command_line_init_writes_a_loadable_folder(tmp_path):
+    """``reinfer init`` with this design's config.json: a folder the engine loads, every declared tensor in it."""
+    from reinfer_amd import cli
+    src = tmp_path / "config.json"
+    src.write_text(json.dumps(PS_A))
+    out = tmp_path / "model"
+    assert cli.main(["init", str(src), "--seed", "3", "--out", str(out), "--dtype", "float32"]) == 0
+    raw, w = read_folder(str(out))
+    assert raw["architecture"] == "Puresun" and raw["layers"][1]["mlp"] is None
+    assert {"embed", "bigram", "loop.step", "l0.norm1", "l0.mix.dkv.norm", "l2.mlp.e2.down", "l0.mlp.router",
+            "final.norm", "head"} <= set(w) and "l1.mlp.router" not in w
+    assert w["loop.step"].shape == (3, 48) and w["bigram"].shape == (98, 48) and w["l1.mix.uk"].shape == (16, 24)
+    with kernels.use(KernelDouble()):
+        eng = LLMEngine(str(out), dtype="float32", device="cpu", num_blocks=16)
+        toks = eng.generate([[1, 2, 3]], SamplingParams(temperature=0.0, max_tokens=4))[0].token_ids
+    assert toks == plain.greedy_generate(raw, w, [1, 2, 3], 4)
+
+
+@pytest.mark.gpu
+def test_command_line_run_gpu(tmp_path):
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = make_folder(tmp_path, "A", "float32")
+    raw, w = read_folder(folder)
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "reinfer"), "run", folder, "-n", "8", "-t", "0",
+                        "--dtype", "float32", "--num-blocks", "16", "--max-model-len", "128", "--", "5", "9", "200"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [int(t) for t in r.stdout.split()] == plain.greedy_generate(raw, w, [5, 9, 200], 8)
