@@ -363,8 +363,8 @@ def _puresun_raw(width, heads, layers, loop, experts, top, ff, window, vocab):
     mixer = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5,
              "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 64}}
     mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
-    raw = {"architecture": "Puresun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
-           "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+    raw = {"architecture": "Puresun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 50.0,
+           "embedding": {"bigram": {"buckets": 65521, "mul_prev": 92821, "mul_cur": 689}},
            "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
     if loop:
         raw["loop"] = {"start": 0, "stop": loop[0], "times": loop[1]}

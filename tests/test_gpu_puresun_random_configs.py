@@ -44,13 +44,13 @@ def rounding_sensitivity(raw, weights, toks, ref):
 
 def draw_config(rng, all_experts: bool):
     n_layers = rng.choice([1, 2, 3, 4])
-    width = rng.choice([40, 72, 100, 136, 264])
+    width = rng.choice([40, 72, 100, 152, 264])
     layers = []
     for _ in range(n_layers):
         dim, rot = rng.choice([8, 16, 24, 40, 64]), rng.choice([2, 4, 8, 16, 32])
         rank = rng.choice([16, 24, 56, 90, 128, 200, 270])
         mixer = ph._mixer(rng.choice([1, 2, 3, 4, 6, 7, 12, 17]), dim, rot, rng.choice([4, 8, 20, 32]), rank,
-                          rng.choice([3, 16, 17, 33, 64, 100, 150]), base=rng.choice([100.0, 10000.0, 5e5]))
+                          rng.choice([3, 16, 17, 33, 64, 100, 150]), base=rng.choice([100.0, 10000.0, 3e5]))
         mlp = None
         if rng.random() < 0.8:
             experts = rng.choice([1, 2, 3, 5, 8, 12])
@@ -60,10 +60,10 @@ def draw_config(rng, all_experts: bool):
     raw = {"architecture": "Puresun", "vocab": rng.choice([131, 333, 1003]), "width": width,
            "norm": {"eps": rng.choice([1e-6, 1e-5, 3e-4])}, "layers": layers}
     if rng.random() < 0.7:
-        raw["logit_softcap"] = rng.choice([5.0, 30.0])
+        raw["logit_softcap"] = rng.choice([5.0, 25.0])
     if rng.random() < 0.7:
-        raw["embedding"] = {"bigram": {"buckets": rng.choice([7, 101, 509]), "mul_prev": rng.choice([1, 31, 1000003]),
-                                       "mul_cur": rng.choice([1, 7, 999983])}}
+        raw["embedding"] = {"bigram": {"buckets": rng.choice([7, 101, 499]), "mul_prev": rng.choice([1, 37, 1000003]),
+                                       "mul_cur": rng.choice([1, 11, 999983])}}
     if rng.random() < 0.7:
         start = rng.randrange(0, n_layers)
         raw["loop"] = {"start": start, "stop": rng.randint(start + 1, n_layers), "times": rng.choice([1, 2, 3])}
