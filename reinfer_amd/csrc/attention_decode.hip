@@ -384,6 +384,27 @@ flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restr
 
 // Workgroups of the kernel that the current device holds at once (asked once a head-size variant, waves a
 // workgroup and LDS size; the answer of the first device stands for all: one kind of GPU in a process).
+// LDS a workgroup may ask for on the current device. Above 64 KB a kernel has to be told so before it is
+// launched or asked about (fd_allow_lds); a device that cannot be asked counts as 64 KB.
+static size_t fd_lds_limit(void) {
+  static size_t cached = 0;
+  if (cached == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && v > 64 * 1024)
+      cached = (size_t)v;
+    else
+      cached = 64 * 1024;
+  }
+  return cached;
+}
+template <int DM, bool EX, int WV>
+static hipError_t fd_allow_lds(size_t lds) {
+  if (lds <= 64 * 1024) return hipSuccess;
+  return hipFuncSetAttribute((const void*)flash_decode_kernel<DM, EX, WV>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                             (int)lds);
+}
+
 static int fd_resident_workgroups(int variant, int waves, size_t lds) {
   static int cached[3][2] = {{0, 0}, {0, 0}, {0, 0}};
   static size_t cached_lds[3][2] = {{0, 0}, {0, 0}, {0, 0}};
@@ -395,6 +416,8 @@ static int fd_resident_workgroups(int variant, int waves, size_t lds) {
   hipError_t e = hipSuccess;
   // the exact form of a head size needs a few registers more than the other: ask for it
 #define RA_FD_OCC(DM)                                                                                                  \
+  e = waves == 4 ? fd_allow_lds<DM, true, 4>(lds) : fd_allow_lds<DM, true, 12>(lds);                                   \
+  if (e == hipSuccess)                                                                                                 \
   e = waves == 4 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<DM, true, 4>, 4 * RA_WAVE, lds) \
                  : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<DM, true, 12>, 12 * RA_WAVE, lds)
   if (variant == 0) RA_FD_OCC(64);
@@ -413,8 +436,10 @@ extern "C" int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_si
   const int G = Hq / Hkv;
   // the waves of a workgroup add their partial results through LDS: the small form (4 waves) must fit
   const size_t lds = (size_t)4 * G * (d + 2) * sizeof(float);
-  return (G >= 1 && G <= 16 && d % 16 == 0 && d >= 16 && d <= 256 && block_size > 0 &&
-          block_size % 16 == 0 && lds <= 64 * 1024) ? 1 : 0;
+  if (!(G >= 1 && G <= 16 && d % 16 == 0 && d >= 16 && d <= 256 && block_size > 0 && block_size % 16 == 0)) return 0;
+  if (lds <= 64 * 1024) return 1;
+  // more than 64 KB (16 heads of 256): where the device gives a workgroup that much and then holds one
+  return (lds <= fd_lds_limit() && fd_resident_workgroups(2, 4, lds) > 0) ? 1 : 0;
 }
 
 // Workgroups of the decode kernel, in its form with `waves` waves a workgroup (4 or 12), that the current
@@ -423,7 +448,7 @@ extern "C" int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_si
 extern "C" int ra_attention_decode_slots(int Hq, int Hkv, int d, int waves) {
   if (!ra_attention_decode_supports(Hq, Hkv, d, 16) || (waves != 4 && waves != 12)) return 0;
   const size_t lds = (size_t)waves * (Hq / Hkv) * (d + 2) * sizeof(float);
-  if (lds > 64 * 1024) return 0;
+  if (lds > 64 * 1024 && !(waves == 4 && lds <= fd_lds_limit())) return 0;
   return fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, waves, lds);
 }
 
@@ -451,17 +476,22 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
   const int G = Hq / Hkv;
   const float scale_log2 = scale * 1.4426950408889634f;
   const size_t lds = (size_t)waves * G * (d + 2) * sizeof(float);
-  RA_CHECK(lds <= 64 * 1024, "attention_decode: %d heads of %d per KV head need too much LDS", G, d);
+  RA_CHECK(lds <= 64 * 1024 || (waves == 4 && lds <= fd_lds_limit()),
+           "attention_decode: %d heads of %d per KV head need too much LDS for workgroups of %d waves", G, d, waves);
   const int slots = fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, waves, lds);
   RA_CHECK(slots > 0, "attention_decode: cannot size the grid (%s)", hipGetErrorString(hipGetLastError()));
   const long items_max = (long)n_tokens * Hkv * max_chunks;
   RA_CHECK(items_max < (1L << 30), "attention_decode: %ld work items in one launch", items_max);
   const int grid = (int)(items_max < slots ? items_max : slots);
 #define RA_FD_GO(DM, EX, WV)                                                                          \
-  flash_decode_kernel<DM, EX, WV><<<grid, WV * RA_WAVE, lds, stream>>>(                               \
-      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
-      (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions, block_size, \
-      Hkv, G, d, scale_log2, window, chunk_shift, max_chunks, n_tokens, 0, part_o, part_ml)
+  do {                                                                                                \
+    if (fd_allow_lds<DM, EX, WV>(lds) != hipSuccess)                                                  \
+      return ra_fail("attention_decode: the device does not give a workgroup %zu bytes of LDS", lds); \
+    flash_decode_kernel<DM, EX, WV><<<grid, WV * RA_WAVE, lds, stream>>>(                             \
+        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                  \
+        (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions, block_size, \
+        Hkv, G, d, scale_log2, window, chunk_shift, max_chunks, n_tokens, 0, part_o, part_ml);        \
+  } while (0)
 #define RA_FD(DM)                                                                                     \
   do {                                                                                                \
     if (waves == 4) {                                                                                 \

@@ -884,6 +884,30 @@ def test_attention_decode(Hq, Hkv, d):
                 close(out, ref, 2 ** -7)     # probabilities and values are bfloat16 products summed in float
 
 
+def test_attention_decode_sixteen_heads_of_256_on_one_kv_head():
+    """The waves' partial results of 16 heads of 256 need 66 KB of LDS, more than a workgroup gets unasked: the small
+    form asks the device for it; where the device gives less, the sizes are refused and the dispatch takes the plain
+    kernel. Either way ``attention`` is right."""
+    from reinfer_amd.kernels import library
+    Hq, Hkv, d = 16, 1, 256
+    flash = bool(library.load().ra_attention_decode_supports(Hq, Hkv, d, 16))
+    for bi, (q_lens, starts) in enumerate(DEC_BATCHES[2:]):
+        for window in (0, 19):
+            q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=40 + bi)
+            batch = FakeBatch(q_lens, starts, tables)
+            T = sum(q_lens)
+            scale = 1.0 / math.sqrt(d)
+            ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
+            out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+            ops().attention(q.view(T, Hq * d), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, scale, window, 0)
+            close(out, ref, 2 ** -7)
+            for chunk in ((None, 128, 1024) if flash else ()):
+                out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+                ops().attention_decode(q.view(T, Hq * d), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, scale, window, 0,
+                                       chunk=chunk, waves=4 if chunk else None)
+                close(out, ref, 2 ** -7)
+
+
 def test_attention_decode_more_tokens_than_one_launch_numbers():
     """The kernel numbers the work items of at most 1024 tokens a launch; longer
     lists go in slices, with and without a token list."""
