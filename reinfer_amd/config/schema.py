@@ -91,6 +91,7 @@ class NormSpec:
     kind: str            # registry name of the norm part, e.g. "rmsnorm"
     size: int
     eps: float
+    offset: float = 0.0  # the stored weight lies around zero: the factor is offset + w (1.0 for "one plus w")
 
 
 @dataclass(frozen=True)
@@ -119,6 +120,7 @@ class MixerSpec:
     bias: bool = False
     position: PositionSpec = PositionSpec("none")
     extra: Tuple[Tuple[str, Any], ...] = ()   # for mixers defined elsewhere
+    value_dim: int = 0              # size of a value head where it differs from head_dim (0: the same)
     # A mixer that is not attention-shaped brings a record of its own (any frozen dataclass) with the
     # sizes and constants it needs, typed as it likes; the fields above then stay at their defaults.
     params: Any = None
@@ -154,11 +156,60 @@ class LatentAttentionSpec:
 class MoESpec:
     """Routing of a mixture-of-experts feed-forward (``FeedForwardSpec.params``; ``intermediate`` is one
     expert's width): ``experts`` of which each token uses ``top``; ``activation`` of an expert ("relu2": the
-    square of relu, no gate); ``weights``: "softmax_chosen" = softmax over the chosen logits alone."""
+    square of relu, no gate; "silu_gated": silu(gate) * up, an expert then has a gate matrix as well);
+    ``weights``: "softmax_chosen" = softmax over the chosen logits alone; "sigmoid" = the sigmoid of each chosen
+    logit times ``weight_scale``, not renormalised. ``groups`` > 1: the experts form that many equal runs of
+    neighbours, a run's score is the sum of its ``group_top`` largest scores, and only experts of the
+    ``groups_kept`` best runs can be chosen. ``shared`` > 0: one more expert of that width, same form, runs
+    for every token with weight 1."""
     experts: int
     top: int
     activation: str = "relu2"
     weights: str = "softmax_chosen"
+    weight_scale: float = 1.0
+    groups: int = 1
+    groups_kept: int = 1
+    group_top: int = 2
+    shared: int = 0
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """A matrix memory with exponential gates (``MixerSpec.params`` of the "matrix_memory" mixer): per head a
+    [key_dim, value_dim] state, a normaliser vector and a running maximum of the log gates; the log input gate
+    and the pre-activation of the forget gate are soft-capped at ``gate_cap`` (0: no cap); ``norm_eps`` is the
+    eps of the per-head norm of the read-out; ``denom_eps`` is added to the read-out's denominator."""
+    heads: int
+    key_dim: int
+    value_dim: int
+    gate_cap: float
+    norm_eps: float
+    denom_eps: float = 1e-6
+
+
+@dataclass(frozen=True)
+class DeltaRuleSpec:
+    """A gated delta rule (``MixerSpec.params`` of the "gated_delta_rule" mixer): ``heads`` value heads of
+    ``value_dim``, ``key_heads`` query/key heads of ``key_dim`` shared by heads // key_heads value heads each, a
+    causal filter of ``conv_taps`` taps over time on q, k and v, ``unit_eps`` inside the root of the unit norm
+    of q and k, ``norm_eps`` of the per-head norm of the read-out."""
+    heads: int
+    key_heads: int
+    key_dim: int
+    value_dim: int
+    conv_taps: int
+    norm_eps: float
+    unit_eps: float = 1e-6
+
+
+@dataclass(frozen=True)
+class SideBySideSpec:
+    """Several mixers on one input (``MixerSpec.params`` of the "side_by_side" mixer): ``members`` are
+    (tensor-name prefix, MixerSpec) pairs; each member's output is RMS-normed over the width (``norm_eps``) with
+    a plain weight ``<prefix><out_name>`` and the results are averaged."""
+    members: Tuple[Tuple[str, Any], ...]
+    norm_eps: float
+    out_name: str = "out"
 
 
 @dataclass(frozen=True)
@@ -207,6 +258,7 @@ class BlockSpec:
     ffn_prefix: str = "mlp."
     mixer_norm_name: str = "input_layernorm.weight"
     ffn_norm_name: str = "post_attention_layernorm.weight"
+    residual_scale: float = 1.0     # x += residual_scale * part(norm(x)) for both parts of the block
     params: Any = None
     extra: Tuple[Tuple[str, Any], ...] = ()
 
@@ -252,6 +304,8 @@ class ModelSpec:
     stream_vectors: Tuple[Tuple[str, int], ...] = ()
     # logits <- cap * tanh(logits / cap) when cap > 0
     logit_softcap: float = 0.0
+    # the embedding rows are multiplied by this on their way into the stream (a tied head uses the table as it is)
+    embed_scale: float = 1.0
 
     def __post_init__(self):
         for i, e in enumerate(self.run_order):

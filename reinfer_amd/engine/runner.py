@@ -16,7 +16,7 @@ from ..cache import CacheManager, OutOfBlocks, plan_groups
 from ..config import load_config
 from ..config.schema import ModelSpec
 from ..models import DecoderModel, declare_params
-from ..parts import KVNeed, LayerCache, PagedNeed, StateNeed
+from ..parts import JointNeed, KVNeed, LayerCache, PagedNeed, StateNeed, paged_need
 from ..weights import check_tensors, load_weights, random_tensor, random_tensors, storage_dtype, weight_from_folder
 from .._hostlib import StepError
 from .batch import StepBatch, StepEntry, build_step_batch
@@ -59,8 +59,8 @@ class ModelRunner:
         # which run-order entries keep keys of their own, and with which window
         windows: List[Optional[int]] = []
         for e, need in zip(spec.run_order, needs):
-            if isinstance(need, (KVNeed, PagedNeed)) and e.cache_from is None:
-                windows.append(need.window)
+            if paged_need(need) is not None and e.cache_from is None:
+                windows.append(paged_need(need).window)
             else:
                 windows.append(None)
         # no layer with keys of its own: no group, no pool, no block tables; requests then hold a state
@@ -78,29 +78,35 @@ class ModelRunner:
         self.manager = CacheManager(groups, self.block_size, [self.num_blocks] * len(groups), max_seqs)
 
         # device side of the cache: what each mixer's need names, a tensor of [blocks, *one block] each
+        def make(need, i) -> Optional[LayerCache]:
+            if isinstance(need, (KVNeed, PagedNeed)):
+                tensors = {}
+                for name, shape, tdtype in need.block_tensors(self.block_size):
+                    tensors[name] = torch.zeros((self.num_blocks, *shape), dtype=tdtype or dtype, device=device)
+                return LayerCache(k=tensors.get("k"), v=tensors.get("v"), group=group_of[i], writes=True,
+                                  tensors=tensors)
+            if isinstance(need, StateNeed):
+                return LayerCache(state=torch.zeros((max_seqs, *need.shape), dtype=need.dtype, device=device))
+            if isinstance(need, JointNeed):
+                return LayerCache(group=group_of.get(i, 0), members=[make(m, i) for m in need.members])
+            return None
+
         self.caches: List[Optional[LayerCache]] = []
         for i, (e, need) in enumerate(zip(spec.run_order, needs)):
-            if isinstance(need, (KVNeed, PagedNeed)):
-                if e.cache_from is None:
-                    tensors = {}
-                    for name, shape, tdtype in need.block_tensors(self.block_size):
-                        tensors[name] = torch.zeros((self.num_blocks, *shape), dtype=tdtype or dtype, device=device)
-                    self.caches.append(LayerCache(k=tensors.get("k"), v=tensors.get("v"), group=group_of[i],
-                                                  writes=True, tensors=tensors))
-                else:
-                    src = self.caches[e.cache_from]
-                    src_need = needs[e.cache_from]
-                    if not isinstance(src_need, (KVNeed, PagedNeed)) or \
-                            tuple(src_need.block_tensors(self.block_size)) != tuple(need.block_tensors(self.block_size)):
-                        raise ValueError(f"run entry {i} cannot read the cache of entry {e.cache_from}: "
-                                         "different heads")
-                    self.caches.append(LayerCache(k=src.k, v=src.v, group=src.group, writes=False,
-                                                  tensors=src.tensors))
-            elif isinstance(need, StateNeed):
-                state = torch.zeros((max_seqs, *need.shape), dtype=need.dtype, device=device)
-                self.caches.append(LayerCache(state=state))
+            if e.cache_from is None:
+                self.caches.append(make(need, i))
+            elif isinstance(need, (KVNeed, PagedNeed)):
+                src = self.caches[e.cache_from]
+                src_need = needs[e.cache_from]
+                if not isinstance(src_need, (KVNeed, PagedNeed)) or \
+                        tuple(src_need.block_tensors(self.block_size)) != tuple(need.block_tensors(self.block_size)):
+                    raise ValueError(f"run entry {i} cannot read the cache of entry {e.cache_from}: "
+                                     "different heads")
+                self.caches.append(LayerCache(k=src.k, v=src.v, group=src.group, writes=False,
+                                              tensors=src.tensors))
             else:
-                self.caches.append(None)
+                raise ValueError(f"run entry {i} cannot read the cache of entry {e.cache_from}: only a layer "
+                                 "that keeps nothing but pages can share them")
 
         # per-request state of the parts at the embedding (one tensor [max_seqs, *shape] each, indexed by the
         # step's state slots like a layer's state)
@@ -189,7 +195,7 @@ class ModelRunner:
         per_block = 0
         for need, w in zip(needs, windows):
             if w is not None:
-                for _, shape, tdtype in need.block_tensors(self.block_size):
+                for _, shape, tdtype in paged_need(need).block_tensors(self.block_size):
                     per_block += math.prod(shape) * torch.empty((), dtype=tdtype or self.dtype).element_size()
         if per_block == 0:
             return 1
@@ -223,11 +229,15 @@ class ModelRunner:
             if not blocks:
                 continue
             idx = torch.tensor(sorted(set(blocks)), dtype=torch.long, device=self.device)
-            for cache in self.caches:
-                if cache is not None and cache.tensors and cache.writes and cache.group == g:
+            for cache in self.paged_caches():
+                if cache.writes and cache.group == g:
                     for t in cache.tensors.values():
                         if t.is_floating_point():
                             t[idx] = float("nan")
+
+    def paged_caches(self) -> List[LayerCache]:
+        """Every cache of the model that holds paged tensors, those of a layer with several mixers included."""
+        return [c for top in self.caches if top is not None for c in top.flat() if c.tensors]
 
     def has_request(self, rid: Hashable) -> bool:
         return rid in self.manager

@@ -121,7 +121,10 @@ class DecoderModel:
         layer by layer the same way, crates/cuda/src/engine.rs:3744-3765)."""
         ops = kernels.current()
         resid = torch.empty((batch.num_tokens, self.spec.hidden), dtype=torch.float32, device=self.device)
-        ops.embed(self.embed, batch.token_ids, resid)
+        if self.spec.embed_scale != 1.0:
+            ops.embed(self.embed, batch.token_ids, resid, scale=float(self.spec.embed_scale))
+        else:
+            ops.embed(self.embed, batch.token_ids, resid)
         if self.input_position is not None:
             self.input_position.add_to_stream(resid, batch)
         for k, part in enumerate(self.inputs):

@@ -7,6 +7,13 @@ projection. Order and formulas: crates/cuda/src/engine.rs:4090-4281 (decode) and
 rotation, scale and cache write and separate calls for prompts and decoding,
 here one fused kernel and one call serve any mix of both. The scale multiplies
 the float score, not q (the reference scales and re-rounds q, engine.rs:4150-4160).
+
+A value head may have a size of its own (``MixerSpec.value_dim``), and head sizes need not be multiples of
+16: the cache and the kernels work on heads of one size D, the larger of the two rounded up to 16, and the
+projections are laid out for it at load (rows of zeros behind each head of W_q, W_k and W_v, columns of zeros
+in W_o). Zeros in q and k add nothing to a score, zeros in v give zeros that W_o's zero columns meet, so
+the result is the attention of the sizes given. Tensor names other than ``q_proj.weight`` ... come as the
+option ``names`` = (q, k, v, o).
 """
 from __future__ import annotations
 
@@ -28,14 +35,20 @@ class GroupedQueryAttention:
     takes_row_scaled = True     # x may be RowScaled: the q/k/v product applies the row factor
     emits_for_norm = True       # forward(..., emit=) may fill a NormTarget from the output projection
 
+    @staticmethod
+    def _names(spec: MixerSpec):
+        return tuple(spec.option("names", ("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight")))
+
     @classmethod
     def declare_params(cls, spec: MixerSpec, prefix: str) -> List[ParamDecl]:
         nq = spec.num_heads * spec.head_dim
         nkv = spec.num_kv_heads * spec.head_dim
-        out = [ParamDecl(prefix + "q_proj.weight", (nq, spec.hidden)),
-               ParamDecl(prefix + "k_proj.weight", (nkv, spec.hidden)),
-               ParamDecl(prefix + "v_proj.weight", (nkv, spec.hidden)),
-               ParamDecl(prefix + "o_proj.weight", (spec.hidden, nq))]
+        vd = spec.value_dim or spec.head_dim
+        q, k, v, o = cls._names(spec)
+        out = [ParamDecl(prefix + q, (nq, spec.hidden)),
+               ParamDecl(prefix + k, (nkv, spec.hidden)),
+               ParamDecl(prefix + v, (spec.num_kv_heads * vd, spec.hidden)),
+               ParamDecl(prefix + o, (spec.hidden, spec.num_heads * vd))]
         if spec.bias:
             out += [ParamDecl(prefix + "q_proj.bias", (nq,), init="zeros", role=MATRIX),
                     ParamDecl(prefix + "k_proj.bias", (nkv,), init="zeros", role=MATRIX),
@@ -51,23 +64,42 @@ class GroupedQueryAttention:
             raise ValueError(f"{spec.num_heads} query heads do not divide into {spec.num_kv_heads} groups")
         self.spec = spec
         self.dtype = dtype
-        self.num_heads, self.num_kv_heads, self.head_dim = spec.num_heads, spec.num_kv_heads, spec.head_dim
+        key_dim, value_dim = spec.head_dim, spec.value_dim or spec.head_dim
+        # the one head size the cache and the kernels work with
+        D = -(-max(key_dim, value_dim) // 16) * 16
+        self.num_heads, self.num_kv_heads, self.head_dim = spec.num_heads, spec.num_kv_heads, D
+        self.key_dim, self.value_dim = key_dim, value_dim
         self.scale = float(spec.scale)
         self.window = int(spec.window)
-        self.qkv_width = (spec.num_heads + 2 * spec.num_kv_heads) * spec.head_dim
+        self.qkv_width = (spec.num_heads + 2 * spec.num_kv_heads) * D
+        qn, kn, vn, on = self._names(spec)
+        if (key_dim != D or value_dim != D) and (spec.qk_norm or spec.bias):
+            raise ValueError("attention: heads that are laid out with zeros behind them take no head norm and no bias")
+
+        def heads_of(w, n, d):           # [n * d, width] -> [n * D, width], zeros behind each head
+            if d == D:
+                return w
+            out = torch.zeros((n, D, w.shape[1]), dtype=w.dtype, device=w.device)
+            out[:, :d] = w.view(n, d, w.shape[1])
+            return out.view(n * D, w.shape[1])
         # rows of q, k, v one after the other: stays [out, in], K contiguous
-        self.w_qkv = torch.cat([weights[prefix + "q_proj.weight"], weights[prefix + "k_proj.weight"],
-                                weights[prefix + "v_proj.weight"]], dim=0).contiguous()
+        self.w_qkv = torch.cat([heads_of(weights[prefix + qn], spec.num_heads, key_dim),
+                                heads_of(weights[prefix + kn], spec.num_kv_heads, key_dim),
+                                heads_of(weights[prefix + vn], spec.num_kv_heads, value_dim)], dim=0).contiguous()
         self.b_qkv = None
         if spec.bias:
             self.b_qkv = torch.cat([weights[prefix + "q_proj.bias"], weights[prefix + "k_proj.bias"],
                                     weights[prefix + "v_proj.bias"]], dim=0).to(dtype).contiguous()
-        self.w_o = weights[prefix + "o_proj.weight"]
+        self.w_o = weights[prefix + on]
+        if value_dim != D:
+            wo = torch.zeros((spec.hidden, spec.num_heads, D), dtype=self.w_o.dtype, device=self.w_o.device)
+            wo[:, :, :value_dim] = self.w_o.view(spec.hidden, spec.num_heads, value_dim)
+            self.w_o = wo.view(spec.hidden, spec.num_heads * D).contiguous()
         self.q_norm = weights[prefix + "q_norm.weight"] if spec.qk_norm else None
         self.k_norm = weights[prefix + "k_norm.weight"] if spec.qk_norm else None
         self.eps = float(spec.qk_norm_eps)
         self.position = lookup("position", spec.position.kind)(spec.position, device)
-        if self.position.rotary_dim > spec.head_dim:
+        if self.position.rotary_dim > key_dim:
             raise ValueError("the rotated width cannot exceed the head size")
 
     def cache_need(self) -> KVNeed:

@@ -46,6 +46,30 @@ class StateNeed:
     dtype: torch.dtype = torch.float32
 
 
+@dataclass(frozen=True)
+class JointNeed:
+    """What a layer keeps when it holds several mixers: each member's own need (None for a member that keeps
+    nothing), in the members' order. At most one member may keep pages (keys and values or other paged
+    tensors): the layer's block tables and window are that member's. The layer's :class:`LayerCache` then
+    has one cache per member in ``members``."""
+    members: Tuple[Optional[object], ...]
+
+    def paged(self):
+        found = [m for m in self.members if isinstance(m, (KVNeed, PagedNeed))]
+        if len(found) > 1:
+            raise ValueError("a layer's mixers may keep pages in one of them only")
+        return found[0] if found else None
+
+
+def paged_need(need):
+    """The part of ``need`` that lives in pages (KVNeed or PagedNeed), or None."""
+    if isinstance(need, (KVNeed, PagedNeed)):
+        return need
+    if isinstance(need, JointNeed):
+        return need.paged()
+    return None
+
+
 @dataclass
 class LayerCache:
     """The cache of one run-order entry, as its mixer sees it.
@@ -63,6 +87,15 @@ class LayerCache:
     writes: bool = True
     state: Optional[torch.Tensor] = None
     tensors: Optional[dict] = None      # every paged tensor by the name its mixer gave it ("k" and "v" among them)
+    members: Optional[list] = None      # for a :class:`JointNeed`: one LayerCache (or None) per member mixer
+
+    def flat(self):
+        """This cache and, for a joint one, its members' caches."""
+        out = [self]
+        for m in self.members or ():
+            if m is not None:
+                out += m.flat()
+        return out
 
 
 @dataclass

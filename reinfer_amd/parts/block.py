@@ -1,7 +1,8 @@
 """How norm, mixer and feed-forward are arranged in a layer.
 
 "prenorm": x += mixer(norm(x)); x += ffn(norm(x))
-(crates/cuda/src/engine.rs:4075-4314). The residual stream is float. A block
+(crates/cuda/src/engine.rs:4075-4314); with ``residual_scale`` s both addends enter times s, and a layer
+may have no feed-forward (then it has no second norm either). The residual stream is float. A block
 gets the stream and the previous block's last addend, not yet added, so that
 the add and the norm are one kernel (the reference fuses the same pair for the
 o-projection, dense_kernels.cu:257-274); it returns its own last addend, or
@@ -26,26 +27,37 @@ class PreNormBlock:
         p = spec.prefix
         out = lookup("norm", spec.mixer_norm.kind).declare_params(spec.mixer_norm, p + spec.mixer_norm_name)
         out += lookup("mixer", spec.mixer.kind).declare_params(spec.mixer, p + spec.mixer_prefix)
-        out += lookup("norm", spec.ffn_norm.kind).declare_params(spec.ffn_norm, p + spec.ffn_norm_name)
-        out += lookup("feed_forward", spec.ffn.kind).declare_params(spec.ffn, p + spec.ffn_prefix)
+        if spec.ffn is not None:
+            out += lookup("norm", spec.ffn_norm.kind).declare_params(spec.ffn_norm, p + spec.ffn_norm_name)
+            out += lookup("feed_forward", spec.ffn.kind).declare_params(spec.ffn, p + spec.ffn_prefix)
         return out
 
     def __init__(self, spec: BlockSpec, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
                  device: torch.device):
-        missing = [n for n in ("mixer", "ffn", "mixer_norm", "ffn_norm") if getattr(spec, n) is None]
+        missing = [n for n in ("mixer", "mixer_norm") if getattr(spec, n) is None]
+        if spec.ffn is not None and spec.ffn_norm is None:
+            missing.append("ffn_norm")
         if missing:
-            raise ValueError(f"a prenorm block is made of a mixer, a feed-forward and a norm before each; "
-                             f"block {spec.prefix!r} names no {', '.join(missing)}")
+            raise ValueError(f"a prenorm block is made of a mixer with a norm before it and at most a feed-forward "
+                             f"with a norm before it; block {spec.prefix!r} names no {', '.join(missing)}")
         p = spec.prefix
         self.spec = spec
         self.mixer_norm = lookup("norm", spec.mixer_norm.kind)(spec.mixer_norm, weights,
                                                                p + spec.mixer_norm_name, dtype, device)
         self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, weights, p + spec.mixer_prefix, dtype, device)
-        self.ffn_norm = lookup("norm", spec.ffn_norm.kind)(spec.ffn_norm, weights,
-                                                           p + spec.ffn_norm_name, dtype, device)
-        self.ffn = lookup("feed_forward", spec.ffn.kind)(spec.ffn, weights, p + spec.ffn_prefix, dtype, device)
+        self.ffn_norm = self.ffn = None
+        if spec.ffn is not None:
+            self.ffn_norm = lookup("norm", spec.ffn_norm.kind)(spec.ffn_norm, weights,
+                                                               p + spec.ffn_norm_name, dtype, device)
+            self.ffn = lookup("feed_forward", spec.ffn.kind)(spec.ffn, weights, p + spec.ffn_prefix, dtype, device)
+        self.residual_scale = float(spec.residual_scale)
+        # the norm-on-products hand-over is for the plain form: both parts there, addends entering as they are
+        self.passes_emit = self.ffn is not None and self.residual_scale == 1.0
 
-    passes_emit = True      # forward(..., emit=) hands a NormTarget on to the feed-forward
+    @property
+    def graph_safe(self) -> bool:
+        return bool(getattr(self.mixer, "graph_safe", False)
+                    and (self.ffn is None or getattr(self.ffn, "graph_safe", False)))
 
     def cache_need(self):
         """What this layer keeps between steps: its mixer's need."""
@@ -53,7 +65,7 @@ class PreNormBlock:
 
     def parts(self):
         """The parts this arrangement is made of (for whoever asks every part something)."""
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None)
 
     def entry_target(self, resid: torch.Tensor):
         """A NormTarget for this block's first norm, for the part that runs before the block, or
@@ -70,6 +82,8 @@ class PreNormBlock:
         # costs no kernel: its column weight is applied by the product before it, its row
         # factor by the product after it.
         mixer, ffn = self.mixer, self.ffn
+        if ffn is None or self.residual_scale != 1.0:
+            return self._forward_scaled(resid, delta, batch, cache)
         xn = self._norm(self.mixer_norm, resid, delta, mixer)
         if getattr(mixer, "adds_in_place", False):
             tgt = self._target(self.ffn_norm, resid, mixer, ffn)
@@ -85,6 +99,31 @@ class PreNormBlock:
                 return ffn.forward(xn, batch, resid=resid, emit=emit)
             return ffn.forward(xn, batch, resid=resid)
         return ffn.forward(xn, batch)
+
+    def _forward_scaled(self, resid: torch.Tensor, delta, batch, cache: Optional[LayerCache]):
+        """x += s * mixer(norm(x)); x += s * ffn(norm(x)), the sums in the float stream. A part that declares
+        ``adds_scaled`` adds s times its result into the stream itself (``forward(..., resid=, resid_scale=)``
+        returns None then); any other part's addend is added by the norm that follows it, or, the block's
+        last one, by the stream-add kernel: this block hands no pending addend on, since whoever adds it
+        would not know its factor."""
+        from .. import kernels
+        s = self.residual_scale
+        if not isinstance(delta, torch.Tensor) and delta is not None:
+            delta = None               # a filled norm target: the sum is already in the stream
+        xn = self.mixer_norm.add_norm(resid, delta)
+        a = self._run(self.mixer, xn, batch, resid, s, cache)
+        if self.ffn is not None:
+            xn = self.ffn_norm.add_norm(resid, a, delta_scale=s) if a is not None else self.ffn_norm.add_norm(resid, None)
+            a = self._run(self.ffn, xn, batch, resid, s)
+        if a is not None:
+            kernels.current().stream_add(resid, a, delta_scale=s)
+        return None
+
+    @staticmethod
+    def _run(part, xn, batch, resid, s, *cache):
+        if getattr(part, "adds_scaled", False):
+            return part.forward(xn, batch, *cache, resid=resid, resid_scale=s)
+        return part.forward(xn, batch, *cache)
 
     @staticmethod
     def _norm(norm, resid, delta, consumer):

@@ -27,17 +27,24 @@ class SwiGLU:
     takes_row_scaled = True     # x may be RowScaled: the gate/up product applies the row factor
     emits_for_norm = True       # forward(..., emit=) may fill a NormTarget from the down projection
 
+    @staticmethod
+    def _names(spec: FeedForwardSpec):
+        """Tensor names of gate, up and down behind the prefix (the option ``names`` where they differ)."""
+        return tuple(dict(spec.extra).get("names", ("gate_proj.weight", "up_proj.weight", "down_proj.weight")))
+
     @classmethod
     def declare_params(cls, spec: FeedForwardSpec, prefix: str) -> List[ParamDecl]:
-        return [ParamDecl(prefix + "gate_proj.weight", (spec.intermediate, spec.hidden)),
-                ParamDecl(prefix + "up_proj.weight", (spec.intermediate, spec.hidden)),
-                ParamDecl(prefix + "down_proj.weight", (spec.hidden, spec.intermediate))]
+        g, u, d = cls._names(spec)
+        return [ParamDecl(prefix + g, (spec.intermediate, spec.hidden)),
+                ParamDecl(prefix + u, (spec.intermediate, spec.hidden)),
+                ParamDecl(prefix + d, (spec.hidden, spec.intermediate))]
 
     def __init__(self, spec: FeedForwardSpec, weights: Dict[str, torch.Tensor], prefix: str,
                  dtype: torch.dtype, device: torch.device):
         self.spec = spec
         self.dtype = dtype
-        gate, up = weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]
+        gn, un, dn = self._names(spec)
+        gate, up = weights[prefix + gn], weights[prefix + un]
         I, h = spec.intermediate, spec.hidden
         self.group = getattr(kernels.current(), "GATE_GROUP", 0)
         if self.group and I % self.group == 0:
@@ -47,7 +54,7 @@ class SwiGLU:
         else:
             self.group = 0
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
-        self.w_down = weights[prefix + "down_proj.weight"]
+        self.w_down = weights[prefix + dn]
 
     def forward(self, x, batch, resid: Optional[torch.Tensor] = None, emit: Optional[NormTarget] = None):
         ops = kernels.current()

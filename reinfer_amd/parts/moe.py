@@ -11,6 +11,15 @@ product with the down matrix is then the weighted sum: with few experts of which
 dense products at the matrix cores' rate cost less than gathering tokens by expert would. A step of so few
 tokens that most experts are not asked for at all (one or two requests decoding) reads only the chosen experts'
 rows instead, a wave a row.
+
+A second form of the same part (``activation`` "silu_gated", ``weights`` "sigmoid"): an expert is
+W_down (silu(W_gate h) * (W_up h)); a token's score for expert e is sigmoid(z_e); where the experts form
+groups of neighbours, a group's score is the sum of its largest scores (two of them) and only experts of the
+best groups can be chosen; the chosen experts' weights are their scores times a constant, not renormalised;
+a shared expert of the same form may run for every token. Here every expert's [gate; up] rows lie one
+after the other in one matrix, the shared expert's behind them, one kernel applies the gate and the
+routing weight (1 for the shared expert, 0 for experts not chosen), and one product with all down
+projections side by side is the sum.
 """
 from __future__ import annotations
 
@@ -33,10 +42,18 @@ class MixtureOfExperts:
     def declare_params(cls, spec: FeedForwardSpec, prefix: str) -> List[ParamDecl]:
         p = spec.params
         out = []
+        gated = p.activation == "silu_gated"
         for e in range(p.experts):
+            if gated:
+                out.append(ParamDecl(f"{prefix}e{e}.gate", (spec.intermediate, spec.hidden)))
             out += [ParamDecl(f"{prefix}e{e}.up", (spec.intermediate, spec.hidden)),
                     ParamDecl(f"{prefix}e{e}.down", (spec.hidden, spec.intermediate))]
         out.append(ParamDecl(prefix + "router", (p.experts, spec.hidden)))
+        if p.shared:
+            if gated:
+                out.append(ParamDecl(prefix + "shared.gate", (p.shared, spec.hidden)))
+            out += [ParamDecl(prefix + "shared.up", (p.shared, spec.hidden)),
+                    ParamDecl(prefix + "shared.down", (spec.hidden, p.shared))]
         return out
 
     def __init__(self, spec: FeedForwardSpec, weights: Dict[str, torch.Tensor], prefix: str,
@@ -44,16 +61,59 @@ class MixtureOfExperts:
         p = spec.params
         if p is None:
             raise ValueError("moe: the routing comes in FeedForwardSpec.params (MoESpec)")
-        if p.activation != "relu2" or p.weights != "softmax_chosen":
+        if (p.activation, p.weights) not in (("relu2", "softmax_chosen"), ("silu_gated", "sigmoid")):
             raise ValueError(f"moe: activation {p.activation!r} with weights {p.weights!r} is not built")
         self.spec = spec
         self.dtype = dtype
         self.experts, self.top, self.ff = int(p.experts), int(p.top), int(spec.intermediate)
+        self.gated = p.activation == "silu_gated"
+        self.routing = p
+        if p.groups < 1 or p.experts % p.groups or not 1 <= p.groups_kept <= p.groups \
+                or p.top > p.groups_kept * (p.experts // p.groups):
+            raise ValueError(f"moe: {p.experts} experts in {p.groups} groups of which {p.groups_kept} are kept "
+                             f"cannot give {p.top} choices")
+        if (p.groups > 1 or p.shared) and not self.gated:
+            raise ValueError("moe: groups of experts and a shared expert are built for the gated form")
+        self.router = weights[prefix + "router"]            # logits are accumulated and kept in float
+        if self.gated:
+            self.shared = int(p.shared)
+            rows = []
+            for e in range(self.experts):
+                rows += [weights[f"{prefix}e{e}.gate"], weights[f"{prefix}e{e}.up"]]
+            downs = [weights[f"{prefix}e{e}.down"] for e in range(self.experts)]
+            if self.shared:
+                rows += [weights[prefix + "shared.gate"], weights[prefix + "shared.up"]]
+                downs.append(weights[prefix + "shared.down"])
+            self.w_gate_up = torch.cat(rows, dim=0).contiguous()       # [2 (E ff + shared), width]
+            self.w_down = torch.cat(downs, dim=1).contiguous()          # [width, E ff + shared]
+            return
         self.w_up = torch.cat([weights[f"{prefix}e{e}.up"] for e in range(self.experts)], dim=0).contiguous()
         self.w_down = torch.cat([weights[f"{prefix}e{e}.down"] for e in range(self.experts)], dim=1).contiguous()
-        self.router = weights[prefix + "router"]            # logits are accumulated and kept in float
+
+    def _forward_gated(self, x, resid):
+        ops = kernels.current()
+        p = self.routing
+        T = x.shape[0]
+        n = self.experts * self.ff + self.shared
+        ids = torch.empty((T, self.top), dtype=torch.int32, device=x.device)
+        weights = torch.empty((T, self.top), dtype=torch.float32, device=x.device)
+        ops.moe_route(x, self.router, self.top, ids, weights, scoring="sigmoid", scale=float(p.weight_scale),
+                      groups=int(p.groups), groups_kept=int(p.groups_kept), group_top=int(p.group_top))
+        gu = torch.empty((T, 2 * n), dtype=self.dtype, device=x.device)
+        ops.linear(x, self.w_gate_up, gu)
+        act = torch.empty((T, n), dtype=self.dtype, device=x.device)
+        ops.moe_silu_gate_scale(gu, act, ids, weights, self.experts, self.ff, self.shared)
+        can_add = getattr(ops, "can_accumulate", None)
+        if resid is not None and can_add and can_add(act, self.w_down):
+            ops.linear_skinny(act, self.w_down, resid, accumulate=True)
+            return None
+        out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
+        ops.linear(act, self.w_down, out)
+        return out
 
     def forward(self, x, batch, resid: Optional[torch.Tensor] = None):
+        if self.gated:
+            return self._forward_gated(x, resid)
         ops = kernels.current()
         T = x.shape[0]
         n = self.experts * self.ff

@@ -27,10 +27,13 @@ class RMSNorm:
         self.size = spec.size
         self.eps = float(spec.eps)
         self.weight = weights[name]
+        if spec.offset:
+            # a weight stored around zero: the factor offset + w is made once, in float
+            self.weight = (weights[name].float() + float(spec.offset)).contiguous()
         self.dtype = dtype
 
     def add_norm(self, resid: torch.Tensor, delta, rows: Optional[torch.Tensor] = None,
-                 scaled_ok: bool = False):
+                 scaled_ok: bool = False, delta_scale: float = 1.0):
         """``resid += delta`` (float, in place) and the norm of the sum.
 
         With ``rows``, only those rows are computed, into a compact result, and
@@ -48,7 +51,10 @@ class RMSNorm:
             delta = None
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=self.dtype, device=resid.device)
-        kernels.current().add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
+        if delta is not None and delta_scale != 1.0:
+            kernels.current().add_rmsnorm(resid, delta, self.weight, self.eps, out, rows, delta_scale=float(delta_scale))
+        else:
+            kernels.current().add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
         return out
 
     def emit_target(self, resid: torch.Tensor, consumer_scales: bool = True) -> Optional[NormTarget]:

@@ -27,18 +27,18 @@ def v_index(off, e, d):
 class KernelDouble:
     name = "cpu-double"
 
-    def embed(self, table, ids, out):
-        out.copy_(table[ids.long()].float())
+    def embed(self, table, ids, out, scale=1.0):
+        out.copy_(table[ids.long()].float() * scale)
 
-    def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None):
+    def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None, delta_scale=1.0):
         if rows is None:
             if delta is not None:
-                resid.add_(delta.float())
+                resid.add_(delta.float() * delta_scale)
             x = resid
         else:
             x = resid[rows.long()]
             if delta is not None:
-                x = x + delta[rows.long()].float()
+                x = x + delta[rows.long()].float() * delta_scale
         rstd = torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps)
         out.copy_((x * rstd * weight.float()).to(out.dtype))
 
@@ -102,9 +102,9 @@ class KernelDouble:
             row = buckets if (pos[t] == 0 or prev < 0) else (prev * mul_prev + ids[t] * mul_cur) % buckets
             resid[t] += table[row].float()
 
-    def stream_add(self, resid, delta=None, other=None, vec=None):
+    def stream_add(self, resid, delta=None, other=None, vec=None, delta_scale=1.0):
         if delta is not None:
-            resid.add_(delta.float())
+            resid.add_(delta.float() * delta_scale)
         if other is not None:
             resid.add_(other)
         if vec is not None:
@@ -160,12 +160,137 @@ class KernelDouble:
                 y = y * torch.sigmoid(gate[:, h * N:(h + 1) * N].float())
             out[:, h * o_head:h * o_head + N] = y.to(out.dtype)
 
+    # ---- recurrent mixers (state in a layout of this stand-in's own: the state is the kernels' private matter)
+    @staticmethod
+    def scan_state_floats(kind, heads, key_dim, value_dim):
+        return heads * key_dim * value_dim + (heads * (key_dim + 1) if kind == "matrix_memory" else 0)
+
+    @staticmethod
+    def _requests(batch):
+        """(first row, rows, state slot, fresh) of every request of the step."""
+        cu, slots, fresh = batch.cu_tokens.tolist(), batch.state_slots.tolist(), batch.fresh.tolist()
+        return [(cu[i], cu[i + 1] - cu[i], slots[i], bool(fresh[i])) for i in range(batch.num_seqs)]
+
+    def matrix_memory_scan(self, proj, q_off, k_off, v_off, gates, gate_bias, state, batch, H, dk, dv, cap, q_scale,
+                           denom_eps, out):
+        p = proj.float()
+        z = gates + gate_bias
+        a_in = cap * torch.tanh(z[:, :H] / cap)
+        b_f = torch.nn.functional.logsigmoid(cap * torch.tanh(z[:, H:] / cap))
+        nS = H * dk * dv
+        for first, rows, slot, fresh in self._requests(batch):
+            if slot < 0:
+                out[first:first + rows] = 0
+                continue
+            st = state[slot]
+            if fresh:
+                st.zero_()
+            S, n, m = st[:nS].view(H, dk, dv), st[nS:nS + H * dk].view(H, dk), st[nS + H * dk:]
+            for t in range(first, first + rows):
+                q = p[t, q_off:q_off + H * dk].view(H, dk) * q_scale
+                k = p[t, k_off:k_off + H * dk].view(H, dk)
+                v = p[t, v_off:v_off + H * dv].view(H, dv)
+                m_new = torch.maximum(b_f[t] + m, a_in[t])
+                keep, take = torch.exp(b_f[t] + m - m_new), torch.exp(a_in[t] - m_new)
+                S.mul_(keep[:, None, None]).add_(take[:, None, None] * k[:, :, None] * v[:, None, :])
+                n.mul_(keep[:, None]).add_(take[:, None] * k)
+                m.copy_(m_new)
+                den = torch.maximum((n * q).sum(-1).abs(), torch.exp(-m)) + denom_eps
+                out[t] = (torch.einsum("hkv,hk->hv", S, q) / den[:, None]).reshape(-1)
+
+    def head_norm_gate(self, read, weight, per_head, gate, kind, eps, H, dv, out):
+        T = read.shape[0]
+        o = read.view(T, H, dv)
+        o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps)
+        o = o * (weight.view(H, dv) if per_head else weight.view(1, dv))
+        g = gate[:, :H * dv].float().view(T, H, dv)
+        g = torch.sigmoid(g) if kind == "sigmoid" else g * torch.sigmoid(g)
+        out.copy_((o * g).reshape(T, H * dv).to(out.dtype))
+
+    def delta_rule_prepare(self, proj, filt, state, conv_off, batch, G, dk, H, dv, taps, unit_eps, q_scale, qkv):
+        C = 2 * G * dk + H * dv
+        x = proj[:, :C].float()
+        for first, rows, slot, fresh in self._requests(batch):
+            if slot < 0:
+                qkv[first:first + rows] = 0
+                continue
+            tail = state[slot, conv_off:conv_off + (taps - 1) * C].view(taps - 1, C)
+            if fresh:
+                tail.zero_()
+            seq = torch.cat([tail, x[first:first + rows]], dim=0)
+            y = sum(seq[j:j + rows] * filt[:, j][None, :] for j in range(taps))
+            y = y * torch.sigmoid(y)
+            q, k = y[:, :G * dk].reshape(rows, G, dk), y[:, G * dk:2 * G * dk].reshape(rows, G, dk)
+            q = q * torch.rsqrt((q * q).sum(-1, keepdim=True) + unit_eps) * q_scale
+            k = k * torch.rsqrt((k * k).sum(-1, keepdim=True) + unit_eps)
+            qkv[first:first + rows] = torch.cat([q.reshape(rows, -1), k.reshape(rows, -1), y[:, 2 * G * dk:]], dim=1)
+            if taps > 1:
+                tail.copy_(seq[rows:].clone())
+
+    def delta_rule_scan(self, qkv, ba, a_log, dt_bias, state, batch, H, G, dk, dv, out):
+        beta = torch.sigmoid(ba[:, :H])
+        decay = torch.exp(-torch.exp(a_log) * torch.nn.functional.softplus(ba[:, H:] + dt_bias))
+        rep = H // G
+        for first, rows, slot, fresh in self._requests(batch):
+            if slot < 0:
+                out[first:first + rows] = 0
+                continue
+            S = state[slot, :H * dk * dv].view(H, dk, dv)
+            if fresh:
+                S.zero_()
+            for t in range(first, first + rows):
+                q = qkv[t, :G * dk].view(G, dk).repeat_interleave(rep, 0)
+                k = qkv[t, G * dk:2 * G * dk].view(G, dk).repeat_interleave(rep, 0)
+                v = qkv[t, 2 * G * dk:].view(H, dv)
+                S.mul_(decay[t][:, None, None])
+                u = beta[t][:, None] * (v - torch.einsum("hkv,hk->hv", S, k))
+                S.add_(k[:, :, None] * u[:, None, :])
+                out[t] = torch.einsum("hkv,hk->hv", S, q).reshape(-1)
+
+    def normed_mean(self, outs, weights, eps, out=None, resid=None, scale=1.0):
+        y = 0
+        for o, w in zip(outs, weights):
+            o = o.float()
+            y = y + o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * w
+        y = y / len(outs)
+        if resid is not None:
+            resid.add_(scale * y)
+        else:
+            out.copy_(y.to(out.dtype))
+
     # ---- mixture of experts
-    def moe_route(self, x, router, top, ids, weights):
+    def moe_route(self, x, router, top, ids, weights, scoring="softmax_chosen", scale=1.0, groups=1, groups_kept=1,
+                  group_top=2):
         z = x.float() @ router.float().T
-        val, idx = torch.topk(z, top, dim=-1)
+        if scoring == "softmax_chosen":
+            val, idx = torch.topk(z, top, dim=-1)
+            ids.copy_(idx.to(torch.int32))
+            weights.copy_(torch.softmax(val, dim=-1))
+            return
+        s = torch.sigmoid(z)
+        T, E = s.shape
+        allowed = s
+        if groups > 1:
+            per = s.view(T, groups, E // groups)
+            gscore = torch.topk(per, min(group_top, E // groups), dim=-1).values.sum(-1)
+            kept = torch.topk(gscore, groups_kept, dim=-1).indices
+            mask = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, kept, True)
+            allowed = torch.where(mask[:, :, None].expand(T, groups, E // groups).reshape(T, E), s,
+                                  torch.full_like(s, -1.0))
+        val, idx = torch.topk(allowed, top, dim=-1)
         ids.copy_(idx.to(torch.int32))
-        weights.copy_(torch.softmax(val, dim=-1))
+        weights.copy_(val * scale)
+
+    def moe_silu_gate_scale(self, gu, act, ids, weights, experts, ff, shared):
+        T = gu.shape[0]
+        p = torch.zeros((T, experts))
+        p.scatter_(1, ids.long(), weights)
+        g = gu[:, :2 * experts * ff].float().view(T, experts, 2, ff)
+        a = (g[:, :, 0] * torch.sigmoid(g[:, :, 0]) * g[:, :, 1] * p[:, :, None]).reshape(T, experts * ff)
+        if shared:
+            sg = gu[:, 2 * experts * ff:].float().view(T, 2, shared)
+            a = torch.cat([a, sg[:, 0] * torch.sigmoid(sg[:, 0]) * sg[:, 1]], dim=1)
+        act.copy_(a.to(act.dtype))
 
     def moe_relu2_scale(self, up, act, ids, weights, experts, ff):
         T = up.shape[0]

@@ -348,8 +348,12 @@ def check_latent(device):
 
 def test_prenorm_block_names_what_it_misses():
     norm = NormSpec("rmsnorm", 48, 1e-6)
-    spec = BlockSpec("prenorm", mixer=_attention(RAW), mixer_norm=norm, prefix="L.")
-    with pytest.raises(ValueError, match="names no ffn, ffn_norm"):
+    # a layer may lack its feed-forward; a feed-forward without the norm before it, or a mixer without one, may not
+    spec = BlockSpec("prenorm", mixer=_attention(RAW), ffn=FeedForwardSpec("swiglu", 48, 96), mixer_norm=norm, prefix="L.")
+    with pytest.raises(ValueError, match="names no ffn_norm"):
+        lookup("block", "prenorm")(spec, {}, torch.float32, torch.device("cpu"))
+    spec = BlockSpec("prenorm", mixer=_attention(RAW), prefix="L.")
+    with pytest.raises(ValueError, match="names no mixer_norm"):
         lookup("block", "prenorm")(spec, {}, torch.float32, torch.device("cpu"))
 
 
