@@ -36,20 +36,20 @@ extern "C" int ra_abi_version(void) { return RA_ABI_VERSION; }
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ out, int h) {
+                             float* __restrict__ out, int h, float scale) {
   const int t = blockIdx.x;
   const T* row = table + (size_t)ids[t] * h;
   float* o = out + (size_t)t * h;
-  for (int i = threadIdx.x; i < h; i += blockDim.x) o[i] = to_f32(row[i]);
+  for (int i = threadIdx.x; i < h; i += blockDim.x) o[i] = to_f32(row[i]) * scale;
 }
 
 extern "C" int ra_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens,
-                        int hidden, hipStream_t stream) {
+                        int hidden, float scale, hipStream_t stream) {
   RA_CHECK(n_tokens > 0 && hidden > 0, "embed: empty input (%d tokens, width %d)", n_tokens, hidden);
   if (table_dtype == RA_F32)
-    embed_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, ids, out, hidden);
+    embed_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, ids, out, hidden, scale);
   else if (table_dtype == RA_BF16)
-    embed_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)table, ids, out, hidden);
+    embed_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)table, ids, out, hidden, scale);
   else
     return ra_fail("embed: unknown dtype tag %d", table_dtype);
   RA_LAUNCH_CHECK("embed");
@@ -66,7 +66,7 @@ extern "C" int ra_embed(const void* table, int table_dtype, const int* ids, floa
 template <typename TA, typename TW>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta,
                                    const TW* __restrict__ w, TA* __restrict__ out,
-                                   const int* __restrict__ rows, int h, float eps) {
+                                   const int* __restrict__ rows, int h, float eps, float dscale) {
   __shared__ float red[17];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -76,7 +76,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
   for (int i = threadIdx.x; i < h; i += blockDim.x) {
     float v = x[i];
     if (dl) {
-      v += to_f32(dl[i]);
+      v += dscale * to_f32(dl[i]);
       if (!rows) x[i] = v;      // the same thread reads it back below
     }
     ss += v * v;
@@ -86,7 +86,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
   TA* o = out + (size_t)r * h;
   for (int i = threadIdx.x; i < h; i += blockDim.x) {
     float v = x[i];
-    if (dl && rows) v += to_f32(dl[i]);
+    if (dl && rows) v += dscale * to_f32(dl[i]);
     o[i] = from_f32<TA>(v * rstd * to_f32(w[i]));
   }
 }
@@ -117,7 +117,7 @@ template <> struct Vec4<bf16_t> {
 template <typename TA, typename TW>
 __global__ void add_rmsnorm_reg_kernel(float* __restrict__ resid, const TA* __restrict__ delta,
                                        const TW* __restrict__ w, TA* __restrict__ out,
-                                       const int* __restrict__ rows, int h, float eps) {
+                                       const int* __restrict__ rows, int h, float eps, float dscale) {
   __shared__ float red[17];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -132,7 +132,7 @@ __global__ void add_rmsnorm_reg_kernel(float* __restrict__ resid, const TA* __re
     wv[j] = v[j];
     if (i < h) {
       v[j] = Vec4<float>::load(x + i);
-      if (dl) v[j] += Vec4<TA>::load(dl + i);
+      if (dl) v[j] += Vec4<TA>::load(dl + i) * dscale;
       wv[j] = Vec4<TW>::load(w + i);
     }
   }
@@ -156,7 +156,7 @@ __global__ void add_rmsnorm_reg_kernel(float* __restrict__ resid, const TA* __re
 
 extern "C" int ra_add_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype,
                               void* out, int act_dtype, const int* rows, int n_rows, int hidden,
-                              float eps, hipStream_t stream) {
+                              float eps, float delta_scale, hipStream_t stream) {
   RA_CHECK(n_rows > 0 && hidden > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_rows, hidden);
   int threads = hidden >= 2048 ? 512 : 256;
   const bool aligned = hidden % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
@@ -171,11 +171,11 @@ extern "C" int ra_add_rmsnorm(float* resid, const void* delta, const void* weigh
   do {                                                                                                 \
     if (in_regs)                                                                                       \
       add_rmsnorm_reg_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(                                  \
-          resid, (const TA*)delta, (const TW*)weight, (TA*)out, rows, hidden, eps);                    \
+          resid, (const TA*)delta, (const TW*)weight, (TA*)out, rows, hidden, eps, delta_scale);       \
     else                                                                                               \
       add_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(resid, (const TA*)delta,             \
                                                                  (const TW*)weight, (TA*)out, rows,    \
-                                                                 hidden, eps);                         \
+                                                                 hidden, eps, delta_scale);            \
   } while (0)
   if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_GO(float, float);
   else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_GO(bf16_t, bf16_t);

@@ -60,6 +60,170 @@ extern "C" int ra_moe_topk(const float* logits, int ld, int experts, int top, in
 }
 
 // ---------------------------------------------------------------------------
+// Sigmoid scores with groups of experts. One wave a token: s_e = sigmoid(z_e) goes to LDS; with more than one
+// group (equal runs of neighbours) a group's score is the sum of its `group_top` largest s, the `kept` groups
+// with the highest scores stay (ties: the lower group) and the experts of the others are struck; then `top`
+// rounds of a wave-wide maximum as above. weights[t, j] = s * scale, not renormalised.
+// ---------------------------------------------------------------------------
+__global__ void moe_route_sigmoid_kernel(const float* __restrict__ logits, int ld, int E, int top, int groups,
+                                         int kept, int group_top, float scale, int* __restrict__ ids,
+                                         float* __restrict__ weights, int T) {
+  extern __shared__ float zs[];          // [MOE_TOPK_WAVES][E + groups]
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE;
+  const int t = blockIdx.x * MOE_TOPK_WAVES + wave;
+  if (t >= T) return;                    // whole waves leave; no workgroup barrier below
+  float* s = zs + (size_t)wave * (E + groups);
+  float* gs = s + E;
+  for (int e = lane; e < E; e += RA_WAVE) s[e] = 1.f / (1.f + expf(-logits[(size_t)t * ld + e]));
+  __builtin_amdgcn_wave_barrier();
+  if (groups > 1) {
+    const int size = E / groups;
+    // a lane scores whole groups: the sum of the group's `group_top` largest, found by striking in a private copy
+    for (int g = lane; g < groups; g += RA_WAVE) {
+      float sum = 0.f;
+      unsigned long long taken = 0ull;       // groups of up to 64 experts mark their taken ones here
+      for (int r = 0; r < group_top && r < size; ++r) {
+        float best = -INFINITY;
+        int at = -1;
+        for (int i = 0; i < size; ++i) {
+          if (size <= 64 && ((taken >> i) & 1ull)) continue;
+          const float v = s[g * size + i];
+          if (v > best) { best = v; at = i; }
+        }
+        sum += best;
+        if (size <= 64) taken |= 1ull << at;
+      }
+      gs[g] = sum;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // keep the best `kept` groups: rounds of a wave-wide maximum over the group scores; a kept group's score
+    // becomes +inf, and what is not +inf at the end is struck
+    for (int j = 0; j < kept; ++j) {
+      float best = -INFINITY;
+      int at = 0x7fffffff;
+      for (int g = lane; g < groups; g += RA_WAVE) {
+        const float v = gs[g];
+        if (v != INFINITY && (at == 0x7fffffff || v > best)) { best = v; at = g; }
+      }
+#pragma unroll
+      for (int m = RA_WAVE / 2; m > 0; m >>= 1) {
+        const float ob = __shfl_xor(best, m, RA_WAVE);
+        const int oa = __shfl_xor(at, m, RA_WAVE);
+        if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+      }
+      if (at < groups && (at & (RA_WAVE - 1)) == lane) gs[at] = INFINITY;
+      __builtin_amdgcn_wave_barrier();
+    }
+    for (int e = lane; e < E; e += RA_WAVE)
+      if (gs[e / size] != INFINITY) s[e] = -INFINITY;
+    __builtin_amdgcn_wave_barrier();
+  }
+  float mine = 0.f;
+  int mine_id = 0;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += RA_WAVE) {      // a lane reads back only what it wrote itself
+      const float v = s[e];
+      if (at == 0x7fffffff || v > best) { best = v; at = e; }
+    }
+#pragma unroll
+    for (int m = RA_WAVE / 2; m > 0; m >>= 1) {
+      const float ob = __shfl_xor(best, m, RA_WAVE);
+      const int oa = __shfl_xor(at, m, RA_WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    if (lane == j) { mine = best * scale; mine_id = at; }
+    if (at < E && (at & (RA_WAVE - 1)) == lane) s[at] = -INFINITY;
+  }
+  if (lane < top) {
+    weights[(size_t)t * top + lane] = mine;
+    ids[(size_t)t * top + lane] = mine_id;
+  }
+}
+
+extern "C" int ra_moe_route_sigmoid(const float* logits, int ld, int experts, int top, int groups, int kept,
+                                    int group_top, float scale, int* ids, float* weights, int n_tokens,
+                                    hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && experts > 0, "moe_route_sigmoid: %d tokens, %d experts", n_tokens, experts);
+  RA_CHECK(groups >= 1 && experts % groups == 0 && kept >= 1 && kept <= groups && group_top >= 1,
+           "moe_route_sigmoid: %d experts in %d groups, %d kept, scored by %d", experts, groups, kept, group_top);
+  RA_CHECK(groups == 1 || experts / groups <= 64 || group_top == 1,
+           "moe_route_sigmoid: groups of %d experts (up to 64)", experts / groups);
+  RA_CHECK(top > 0 && top <= RA_WAVE && top <= kept * (experts / groups),
+           "moe_route_sigmoid: %d of %d experts that can be chosen (at most 64)", top, kept * (experts / groups));
+  RA_CHECK(ld >= experts, "moe_route_sigmoid: rows of %d for %d experts", ld, experts);
+  const size_t lds = (size_t)MOE_TOPK_WAVES * (experts + groups) * sizeof(float);
+  RA_CHECK(lds <= 64 * 1024, "moe_route_sigmoid: %d experts", experts);
+  const int blocks = (n_tokens + MOE_TOPK_WAVES - 1) / MOE_TOPK_WAVES;
+  moe_route_sigmoid_kernel<<<blocks, MOE_TOPK_WAVES * RA_WAVE, lds, stream>>>(logits, ld, experts, top, groups, kept,
+                                                                              group_top, scale, ids, weights, n_tokens);
+  RA_LAUNCH_CHECK("moe_route_sigmoid");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Gated experts side by side: gu[t, e * 2 ff + j] is expert e's gate projection of token t and
+// gu[t, e * 2 ff + ff + j] its up projection; behind the experts a shared expert's [gate | up] of `shared` each.
+// act[t, e * ff + j] = p(t, e) * silu(gate) * up for the chosen experts and 0 for the others;
+// act[t, E * ff + j] = silu(gate) * up of the shared expert.
+// ---------------------------------------------------------------------------
+template <typename TA>
+__global__ void moe_silu_gate_scale_kernel(const TA* __restrict__ gu, TA* __restrict__ act,
+                                           const int* __restrict__ ids, const float* __restrict__ weights, int top,
+                                           int E, int ff, int shared) {
+  extern __shared__ float gate[];        // [E]
+  const int t = blockIdx.y;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) gate[e] = 0.f;
+  __syncthreads();
+  for (int j = threadIdx.x; j < top; j += blockDim.x) gate[ids[(size_t)t * top + j]] = weights[(size_t)t * top + j];
+  __syncthreads();
+  const int n = E * ff + shared;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const TA* row = gu + (size_t)t * 2 * n;
+  float p, g, u;
+  if (i < E * ff) {
+    const int e = i / ff, j = i - e * ff;
+    p = gate[e];
+    if (p == 0.f) {
+      act[(size_t)t * n + i] = from_f32<TA>(0.f);
+      return;
+    }
+    g = to_f32(row[(size_t)e * 2 * ff + j]);
+    u = to_f32(row[(size_t)e * 2 * ff + ff + j]);
+  } else {
+    const int j = i - E * ff;
+    p = 1.f;
+    g = to_f32(row[(size_t)E * 2 * ff + j]);
+    u = to_f32(row[(size_t)E * 2 * ff + shared + j]);
+  }
+  act[(size_t)t * n + i] = from_f32<TA>(p * (g / (1.f + expf(-g))) * u);
+}
+
+extern "C" int ra_moe_silu_gate_scale(const void* gu, void* act, int act_dtype, const int* ids, const float* weights,
+                                      int top, int experts, int ff, int shared, int n_tokens, hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && experts > 0 && ff > 0 && top > 0 && top <= experts && shared >= 0,
+           "moe_silu_gate_scale: %d tokens, %d of %d experts of %d, shared %d", n_tokens, top, experts, ff, shared);
+  RA_CHECK(n_tokens <= 65535, "moe_silu_gate_scale: %d tokens in one launch (max 65535)", n_tokens);
+  const size_t lds = (size_t)experts * sizeof(float);
+  RA_CHECK(lds <= 64 * 1024, "moe_silu_gate_scale: %d experts", experts);
+  const int n = experts * ff + shared;
+  dim3 grid((n + 255) / 256, n_tokens);
+  if (act_dtype == RA_F32)
+    moe_silu_gate_scale_kernel<float><<<grid, 256, lds, stream>>>((const float*)gu, (float*)act, ids, weights, top,
+                                                                   experts, ff, shared);
+  else if (act_dtype == RA_BF16)
+    moe_silu_gate_scale_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)gu, (bf16_t*)act, ids, weights, top,
+                                                                    experts, ff, shared);
+  else
+    return ra_fail("moe_silu_gate_scale: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("moe_silu_gate_scale");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Experts side by side: up[t, e * ff + j] is expert e's up projection of token t. act[t, e * ff + j] =
 // p(t, e) * relu(up)^2 for the chosen experts, 0 for the others, so that one product with the down
 // projections laid side by side, [width, E * ff], is the weighted sum of the chosen experts' outputs.

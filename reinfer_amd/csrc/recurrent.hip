@@ -1,0 +1,554 @@
+// Recurrent token mixers: a matrix memory with exponential gates and a gated delta rule, both a float matrix
+// state [key_dim, value_dim] a head that is carried from token to token, and the row kernels around them
+// (gate preparation, the short causal filter with its unit norms, the per-head norm and output gate, the mean of
+// several mixers' normed outputs). Everything here computes in float whatever the activations' type.
+//
+// The scans. A column of the state (one value index) evolves on its own given the token's k, q and gates, so
+// the columns are spread over lanes, waves and workgroups and every wave walks the request's tokens in order:
+// R lanes share a column, lane r of them holding elements r, r + R, ... of it (NPL a lane); a wave holds
+// 64 / R columns. The two dot products a token needs (with k or n, and with q) are sums over a lane's elements
+// and a butterfly over the R lanes. The next token's operands are asked for before the current token's
+// arithmetic. The state of a request lives in its slot in the waves' own order, [NPL][64] floats a wave, so
+// that loading and storing it are whole lines; nothing else reads it.
+#include "common.h"
+#include "reinfer_hip.h"
+
+namespace {
+
+struct ScanGeom {
+  int R, NPL, CPW, waves;      // lanes a column, elements a lane, columns a wave, waves a head
+  int wave_floats;             // floats of state a wave
+};
+
+// kind 0: matrix memory (S, the normaliser n once a wave, the running maximum m); kind 1: delta rule (S)
+bool scan_geom(int kind, int dk, int dv, ScanGeom* g) {
+  if (dk <= 0 || dv <= 0 || dk > 512) return false;
+  g->R = dk <= 128 ? 8 : 32;
+  const int per = (dk + g->R - 1) / g->R;
+  g->NPL = per <= 2 ? 2 : per <= 4 ? 4 : per <= 8 ? 8 : 16;
+  g->CPW = RA_WAVE / g->R;
+  g->waves = (dv + g->CPW - 1) / g->CPW;
+  g->wave_floats = g->NPL * RA_WAVE + (kind == 0 ? g->NPL * g->R + 4 : 0);
+  return true;
+}
+
+template <int R>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int m = R / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, RA_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+__device__ __forceinline__ float logsigmoid_f(float x) { return -softplus_f(-x); }
+
+// ---------------------------------------------------------------------------
+// Matrix memory. lg[t, h] = log input gate a, lg[t, H + h] = log forget gate b (prepared below).
+//   m' = max(b + m, a);  keep = exp(b + m - m');  take = exp(a - m')
+//   S <- keep S + take k v^T;  n <- keep n + take k;  o = S^T q / (max(|n . q|, exp(-m')) + eps)
+// ---------------------------------------------------------------------------
+template <typename TA, int R, int NPL>
+__global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
+    const TA* __restrict__ proj, int ld, int q_off, int k_off, int v_off, const float* __restrict__ lg,
+    float* __restrict__ state, long slot_stride, const int* __restrict__ cu_tokens,
+    const int* __restrict__ state_slots, const int* __restrict__ fresh, int H, int dk, int dv, int waves_per_head,
+    int wave_floats, float q_scale, float denom_eps, float* __restrict__ out) {
+  constexpr int CPW = RA_WAVE / R;
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int w = blockIdx.z * (blockDim.x / RA_WAVE) + threadIdx.x / RA_WAVE;
+  if (w >= waves_per_head) return;           // whole waves leave; there is no barrier below
+  const int c = lane / R, r = lane % R;
+  const int col = w * CPW + c;
+  const bool col_ok = col < dv;
+  const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+  const int slot = state_slots[seq];
+  const int ow = H * dv;
+  if (slot < 0) {                            // a padding row: no state, a defined result
+    if (col_ok && r == 0)
+      for (int t = first; t < last; ++t) out[(size_t)t * ow + head * dv + col] = 0.f;
+    return;
+  }
+  if (first >= last) return;
+  float* st = state + (size_t)slot * slot_stride + (size_t)(head * waves_per_head + w) * wave_floats;
+  const bool zero = fresh[seq] != 0;
+  float S[NPL], n[NPL];
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) {
+    S[i] = zero ? 0.f : st[i * RA_WAVE + lane];
+    n[i] = zero ? 0.f : st[NPL * RA_WAVE + i * R + r];
+  }
+  float m = zero ? 0.f : st[NPL * RA_WAVE + NPL * R];
+  const TA* qp = proj + q_off + head * dk;
+  const TA* kp = proj + k_off + head * dk;
+  const TA* vp = proj + v_off + head * dv + (col_ok ? col : 0);
+  float nk[NPL], nq[NPL], nv, na, nb;
+  auto fetch = [&](int t) {
+    const size_t row = (size_t)t * ld;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const int e = i * R + r;
+      nk[i] = e < dk ? to_f32(kp[row + e]) : 0.f;
+      nq[i] = e < dk ? to_f32(qp[row + e]) : 0.f;
+    }
+    nv = col_ok ? to_f32(vp[row]) : 0.f;
+    na = lg[(size_t)t * 2 * H + head];
+    nb = lg[(size_t)t * 2 * H + H + head];
+  };
+  fetch(first);
+  for (int t = first; t < last; ++t) {
+    float k[NPL], q[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) { k[i] = nk[i]; q[i] = nq[i] * q_scale; }
+    const float v = nv, a = na, b = nb;
+    if (t + 1 < last) fetch(t + 1);
+    const float m_new = fmaxf(b + m, a);
+    const float keep = expf(b + m - m_new);
+    const float take = expf(a - m_new);
+    m = m_new;
+    float ps = 0.f, pn = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const float tk = take * k[i];
+      n[i] = keep * n[i] + tk;
+      S[i] = keep * S[i] + tk * v;
+      ps += S[i] * q[i];
+      pn += n[i] * q[i];
+    }
+    ps = group_sum<R>(ps);
+    pn = group_sum<R>(pn);
+    const float den = fmaxf(fabsf(pn), expf(-m)) + denom_eps;
+    if (col_ok && r == 0) out[(size_t)t * ow + head * dv + col] = ps / den;
+  }
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) {
+    st[i * RA_WAVE + lane] = S[i];
+    if (c == 0) st[NPL * RA_WAVE + i * R + r] = n[i];
+  }
+  if (lane == 0) st[NPL * RA_WAVE + NPL * R] = m;
+}
+
+// lg[t, h] <- cap tanh((z + bias) / cap);  lg[t, H + h] <- log sigmoid(cap tanh((z + bias) / cap)), in place
+__global__ void matrix_memory_gates_kernel(float* __restrict__ lg, const float* __restrict__ bias, int H, float cap,
+                                           long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int j = (int)(i % (2 * H));
+  float z = lg[i] + bias[j];
+  if (cap > 0.f) z = cap * tanhf(z / cap);
+  lg[i] = j < H ? z : logsigmoid_f(z);
+}
+
+// ---------------------------------------------------------------------------
+// Gated delta rule. gb[t, h] = beta, gb[t, H + h] = decay g (prepared below); qkv float [T, q | k | v].
+//   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// computed from the state before the decay: a = S^T k, b = S^T q, kq = k . q in one butterfly, then
+// u = beta (v - g a), o = g b + u kq, S <- g S + k u.
+// ---------------------------------------------------------------------------
+template <int R, int NPL>
+__global__ __launch_bounds__(256) void delta_rule_scan_kernel(
+    const float* __restrict__ qkv, int ld, const float* __restrict__ gb, float* __restrict__ state, long slot_stride,
+    const int* __restrict__ cu_tokens, const int* __restrict__ state_slots, const int* __restrict__ fresh, int H,
+    int G, int dk, int dv, int waves_per_head, float* __restrict__ out) {
+  constexpr int CPW = RA_WAVE / R;
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int w = blockIdx.z * (blockDim.x / RA_WAVE) + threadIdx.x / RA_WAVE;
+  if (w >= waves_per_head) return;
+  const int c = lane / R, r = lane % R;
+  const int col = w * CPW + c;
+  const bool col_ok = col < dv;
+  const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+  const int slot = state_slots[seq];
+  const int ow = H * dv;
+  if (slot < 0) {
+    if (col_ok && r == 0)
+      for (int t = first; t < last; ++t) out[(size_t)t * ow + head * dv + col] = 0.f;
+    return;
+  }
+  if (first >= last) return;
+  float* st = state + (size_t)slot * slot_stride + (size_t)(head * waves_per_head + w) * (NPL * RA_WAVE);
+  const bool zero = fresh[seq] != 0;
+  float S[NPL];
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) S[i] = zero ? 0.f : st[i * RA_WAVE + lane];
+  const int kh = head / (H / G);
+  const float* qp = qkv + kh * dk;
+  const float* kp = qkv + G * dk + kh * dk;
+  const float* vp = qkv + 2 * G * dk + head * dv + (col_ok ? col : 0);
+  float nk[NPL], nq[NPL], nv, nbeta, ng;
+  auto fetch = [&](int t) {
+    const size_t row = (size_t)t * ld;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const int e = i * R + r;
+      nk[i] = e < dk ? kp[row + e] : 0.f;
+      nq[i] = e < dk ? qp[row + e] : 0.f;
+    }
+    nv = col_ok ? vp[row] : 0.f;
+    nbeta = gb[(size_t)t * 2 * H + head];
+    ng = gb[(size_t)t * 2 * H + H + head];
+  };
+  fetch(first);
+  for (int t = first; t < last; ++t) {
+    float k[NPL], q[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) { k[i] = nk[i]; q[i] = nq[i]; }
+    const float v = nv, beta = nbeta, g = ng;
+    if (t + 1 < last) fetch(t + 1);
+    float pa = 0.f, pb = 0.f, pkq = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      pa += S[i] * k[i];
+      pb += S[i] * q[i];
+      pkq += k[i] * q[i];
+    }
+    pa = group_sum<R>(pa);
+    pb = group_sum<R>(pb);
+    pkq = group_sum<R>(pkq);
+    const float u = beta * (v - g * pa);
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) S[i] = g * S[i] + k[i] * u;
+    if (col_ok && r == 0) out[(size_t)t * ow + head * dv + col] = g * pb + u * pkq;
+  }
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) st[i * RA_WAVE + lane] = S[i];
+}
+
+// gb[t, h] <- sigmoid(b);  gb[t, H + h] <- exp(-exp(A_log[h]) softplus(a + dt_bias[h])), in place
+__global__ void delta_rule_gates_kernel(float* __restrict__ gb, const float* __restrict__ a_log,
+                                        const float* __restrict__ dt_bias, int H, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int j = (int)(i % (2 * H));
+  const float z = gb[i];
+  if (j < H) gb[i] = 1.f / (1.f + expf(-z));
+  else gb[i] = expf(-expf(a_log[j - H]) * softplus_f(z + dt_bias[j - H]));
+}
+
+// ---------------------------------------------------------------------------
+// The delta rule's inputs: per channel a causal filter over time (taps weights, the last one the current
+// token's; rows before the step's portion come from the request's tail of taps - 1 rows, zeros at a request's
+// start), silu, and for the heads of q and k the unit norm x / sqrt(sum x^2 + eps) (q also times q_scale).
+// One wave a (token, head of q, k or v); float results [T, C].
+// ---------------------------------------------------------------------------
+#define PREP_WAVES 4
+#define PREP_HOLD 8          // values a lane keeps: heads up to 512 wide
+template <typename TA>
+__global__ void delta_rule_prepare_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ filt,
+                                          const float* __restrict__ state, long slot_stride, long tail_off,
+                                          const int* __restrict__ seq_of_token, const int* __restrict__ cu_tokens,
+                                          const int* __restrict__ state_slots, const int* __restrict__ fresh, int G,
+                                          int dk, int H, int dv, int taps, float unit_eps, float q_scale,
+                                          float* __restrict__ qkv, int T) {
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int units = 2 * G + H;
+  const long idx = (long)blockIdx.x * PREP_WAVES + threadIdx.x / RA_WAVE;
+  if (idx >= (long)T * units) return;
+  const int t = (int)(idx / units), unit = (int)(idx % units);
+  const int C = 2 * G * dk + H * dv;
+  const bool is_v = unit >= 2 * G;
+  const int width = is_v ? dv : dk;
+  const int base = is_v ? 2 * G * dk + (unit - 2 * G) * dv : unit * dk;
+  const int seq = seq_of_token[t];
+  const int first = cu_tokens[seq];
+  const int slot = state_slots[seq];
+  float* o = qkv + (size_t)t * C + base;
+  if (slot < 0) {
+    for (int e = lane; e < width; e += RA_WAVE) o[e] = 0.f;
+    return;
+  }
+  const bool zero = fresh[seq] != 0;
+  const float* tail = state + (size_t)slot * slot_stride + tail_off;      // [taps - 1, C], oldest first
+  float y[PREP_HOLD];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < PREP_HOLD; ++j) {
+    const int e = lane + j * RA_WAVE;
+    y[j] = 0.f;
+    if (e < width) {
+      const int ch = base + e;
+      float acc = 0.f;
+      for (int p = 0; p < taps; ++p) {
+        const int rel = t - first - (taps - 1) + p;        // row of the portion, negative: a row of the tail
+        float x;
+        if (rel >= 0) x = to_f32(proj[(size_t)(first + rel) * ld + ch]);
+        else x = zero ? 0.f : tail[(size_t)(taps - 1 + rel) * C + ch];
+        acc += filt[(size_t)ch * taps + p] * x;
+      }
+      acc = acc / (1.f + expf(-acc));
+      y[j] = acc;
+      ss += acc * acc;
+    }
+  }
+  float f = 1.f;
+  if (!is_v) {
+    ss = wave_sum(ss);
+    f = 1.f / sqrtf(ss + unit_eps);
+    if (unit < G) f *= q_scale;
+  }
+#pragma unroll
+  for (int j = 0; j < PREP_HOLD; ++j) {
+    const int e = lane + j * RA_WAVE;
+    if (e < width) o[e] = y[j] * f;
+  }
+}
+
+// The tail moves on: after a portion of n rows it holds the last taps - 1 rows of (old tail, portion).
+// One thread a (request, channel) reads what it needs before it writes.
+#define MAX_TAPS 16
+template <typename TA>
+__global__ void delta_rule_tail_kernel(const TA* __restrict__ proj, int ld, float* __restrict__ state,
+                                       long slot_stride, long tail_off, const int* __restrict__ cu_tokens,
+                                       const int* __restrict__ state_slots, const int* __restrict__ fresh, int C,
+                                       int taps) {
+  const int seq = blockIdx.y;
+  const int ch = blockIdx.x * blockDim.x + threadIdx.x;
+  if (ch >= C) return;
+  const int slot = state_slots[seq];
+  if (slot < 0) return;
+  const int first = cu_tokens[seq], n = cu_tokens[seq + 1] - first;
+  const bool zero = fresh[seq] != 0;
+  float* tail = state + (size_t)slot * slot_stride + tail_off;
+  float keep[MAX_TAPS];
+  for (int j = 0; j < taps - 1; ++j) {
+    const int rel = n - (taps - 1) + j;
+    if (rel >= 0) keep[j] = to_f32(proj[(size_t)(first + rel) * ld + ch]);
+    else keep[j] = zero ? 0.f : tail[(size_t)(j + n) * C + ch];
+  }
+  for (int j = 0; j < taps - 1; ++j) tail[(size_t)j * C + ch] = keep[j];
+}
+
+// ---------------------------------------------------------------------------
+// out[t, h, :] = read[t, h, :] / rms(read[t, h, :]) * weight * act(gate[t, h, :]); act = sigmoid or silu;
+// weight is [heads * dv] (w_head_stride = dv) or one [dv] for all heads (0). One wave a (token, head).
+// ---------------------------------------------------------------------------
+template <typename TA>
+__global__ void head_norm_gate_kernel(const float* __restrict__ read, const float* __restrict__ weight,
+                                      int w_head_stride, const TA* __restrict__ gate, int ldg, int silu, float eps,
+                                      int H, int dv, TA* __restrict__ out, long n_units) {
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const long idx = (long)blockIdx.x * (blockDim.x / RA_WAVE) + threadIdx.x / RA_WAVE;
+  if (idx >= n_units) return;
+  const long t = idx / H;
+  const int h = (int)(idx % H);
+  const float* x = read + (size_t)t * H * dv + (size_t)h * dv;
+  float ss = 0.f;
+  for (int e = lane; e < dv; e += RA_WAVE) ss += x[e] * x[e];
+  ss = wave_sum(ss);
+  const float rstd = 1.f / sqrtf(ss / (float)dv + eps);
+  const TA* g = gate + (size_t)t * ldg + (size_t)h * dv;
+  const float* wt = weight + (size_t)h * w_head_stride;
+  TA* o = out + (size_t)t * H * dv + (size_t)h * dv;
+  for (int e = lane; e < dv; e += RA_WAVE) {
+    const float z = to_f32(g[e]);
+    const float s = 1.f / (1.f + expf(-z));
+    o[e] = from_f32<TA>(x[e] * rstd * wt[e] * (silu ? z * s : s));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// y[t, :] = (1 / n) sum_i x_i[t, :] / rms(x_i[t, :]) * w_i;  out = y, or resid += scale * y. One workgroup a row.
+// ---------------------------------------------------------------------------
+#define MEAN_MAX 4
+struct MeanInputs {
+  const void* x[MEAN_MAX];
+  const float* w[MEAN_MAX];
+};
+template <typename TA>
+__global__ void normed_mean_kernel(MeanInputs in, int n, float eps, int h, TA* __restrict__ out,
+                                   float* __restrict__ resid, float scale) {
+  __shared__ float red[17];
+  const size_t row = (size_t)blockIdx.x * h;
+  float rstd[MEAN_MAX];
+  for (int i = 0; i < n; ++i) {
+    const TA* x = (const TA*)in.x[i] + row;
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < h; e += blockDim.x) {
+      const float v = to_f32(x[e]);
+      ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    rstd[i] = 1.f / sqrtf(ss / (float)h + eps);
+  }
+  const float inv = 1.f / (float)n;
+  for (int e = threadIdx.x; e < h; e += blockDim.x) {
+    float y = 0.f;
+    for (int i = 0; i < n; ++i) y += to_f32(((const TA*)in.x[i])[row + e]) * rstd[i] * in.w[i][e];
+    y *= inv;
+    if (resid) resid[row + e] += scale * y;
+    else out[row + e] = from_f32<TA>(y);
+  }
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+extern "C" long ra_scan_state_floats(int kind, int heads, int key_dim, int value_dim) {
+  ScanGeom g;
+  if (heads <= 0 || !scan_geom(kind, key_dim, value_dim, &g)) return -1;
+  return (long)heads * g.waves * g.wave_floats;
+}
+
+namespace {
+struct ScanLaunch {
+  dim3 grid;
+  int threads;
+};
+ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads) {
+  const int wpb = g.waves < 4 ? g.waves : 4;           // waves a workgroup
+  ScanLaunch L;
+  L.threads = wpb * RA_WAVE;
+  L.grid = dim3(n_seqs, heads, (g.waves + wpb - 1) / wpb);
+  return L;
+}
+}  // namespace
+
+extern "C" int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, int q_off, int k_off, int v_off,
+                                     float* gates, const float* gate_bias, float* state, long slot_stride,
+                                     const int* cu_tokens, const int* state_slots, const int* fresh, int n_seqs,
+                                     int n_tokens, int heads, int key_dim, int value_dim, float gate_cap,
+                                     float q_scale, float denom_eps, float* out, hipStream_t stream) {
+  RA_CHECK(n_seqs > 0 && n_tokens > 0 && heads > 0, "matrix_memory_scan: %d requests, %d tokens, %d heads", n_seqs,
+           n_tokens, heads);
+  ScanGeom g;
+  RA_CHECK(scan_geom(0, key_dim, value_dim, &g), "matrix_memory_scan: heads of %d x %d (keys up to 512)", key_dim,
+           value_dim);
+  RA_CHECK(slot_stride >= (long)heads * g.waves * g.wave_floats, "matrix_memory_scan: a state slot of %ld floats, need %ld",
+           slot_stride, (long)heads * g.waves * g.wave_floats);
+  RA_CHECK(heads <= 65535, "matrix_memory_scan: %d heads in one launch", heads);
+  const long n = (long)n_tokens * 2 * heads;
+  matrix_memory_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(gates, gate_bias, heads, gate_cap, n);
+  RA_LAUNCH_CHECK("matrix_memory_gates");
+  const ScanLaunch L = scan_launch(g, n_seqs, heads);
+#define RA_MM(TA, R, NPL)                                                                                         \
+  matrix_memory_scan_kernel<TA, R, NPL><<<L.grid, L.threads, 0, stream>>>(                                        \
+      (const TA*)proj, ld, q_off, k_off, v_off, gates, state, slot_stride, cu_tokens, state_slots, fresh, heads,  \
+      key_dim, value_dim, g.waves, g.wave_floats, q_scale, denom_eps, out)
+#define RA_MM_N(TA, R)                                  \
+  do {                                                  \
+    if (g.NPL == 2) RA_MM(TA, R, 2);                    \
+    else if (g.NPL == 4) RA_MM(TA, R, 4);               \
+    else if (g.NPL == 8) RA_MM(TA, R, 8);               \
+    else RA_MM(TA, R, 16);                              \
+  } while (0)
+  if (act_dtype == RA_F32) {
+    if (g.R == 8) RA_MM_N(float, 8); else RA_MM_N(float, 32);
+  } else if (act_dtype == RA_BF16) {
+    if (g.R == 8) RA_MM_N(bf16_t, 8); else RA_MM_N(bf16_t, 32);
+  } else {
+    return ra_fail("matrix_memory_scan: unknown dtype tag %d", act_dtype);
+  }
+#undef RA_MM_N
+#undef RA_MM
+  RA_LAUNCH_CHECK("matrix_memory_scan");
+  return 0;
+}
+
+extern "C" int ra_delta_rule_prepare(const void* proj, int act_dtype, int ld, const float* filt, float* state,
+                                     long slot_stride, long tail_off, const int* seq_of_token, const int* cu_tokens,
+                                     const int* state_slots, const int* fresh, int n_seqs, int n_tokens,
+                                     int key_heads, int key_dim, int heads, int value_dim, int taps, float unit_eps,
+                                     float q_scale, float* qkv, hipStream_t stream) {
+  RA_CHECK(n_seqs > 0 && n_tokens > 0 && heads > 0 && key_heads > 0, "delta_rule_prepare: %d requests, %d tokens",
+           n_seqs, n_tokens);
+  RA_CHECK(taps >= 1 && taps <= MAX_TAPS, "delta_rule_prepare: a filter of %d taps (1 to %d)", taps, MAX_TAPS);
+  RA_CHECK(key_dim <= PREP_HOLD * RA_WAVE && value_dim <= PREP_HOLD * RA_WAVE,
+           "delta_rule_prepare: heads of %d / %d (up to %d)", key_dim, value_dim, PREP_HOLD * RA_WAVE);
+  const int C = 2 * key_heads * key_dim + heads * value_dim;
+  RA_CHECK(slot_stride >= tail_off + (long)(taps - 1) * C, "delta_rule_prepare: a state slot of %ld floats", slot_stride);
+  RA_CHECK(n_seqs <= 65535, "delta_rule_prepare: %d requests in one launch", n_seqs);
+  const long units = (long)n_tokens * (2 * key_heads + heads);
+  const unsigned blocks = (unsigned)((units + PREP_WAVES - 1) / PREP_WAVES);
+  dim3 tail_grid((C + 255) / 256, n_seqs);
+#define RA_DP(TA)                                                                                                   \
+  do {                                                                                                              \
+    delta_rule_prepare_kernel<TA><<<blocks, PREP_WAVES * RA_WAVE, 0, stream>>>(                                     \
+        (const TA*)proj, ld, filt, state, slot_stride, tail_off, seq_of_token, cu_tokens, state_slots, fresh,       \
+        key_heads, key_dim, heads, value_dim, taps, unit_eps, q_scale, qkv, n_tokens);                              \
+    if (taps > 1)                                                                                                   \
+      delta_rule_tail_kernel<TA><<<tail_grid, 256, 0, stream>>>((const TA*)proj, ld, state, slot_stride, tail_off,  \
+                                                                cu_tokens, state_slots, fresh, C, taps);            \
+  } while (0)
+  if (act_dtype == RA_F32) RA_DP(float);
+  else if (act_dtype == RA_BF16) RA_DP(bf16_t);
+  else return ra_fail("delta_rule_prepare: unknown dtype tag %d", act_dtype);
+#undef RA_DP
+  RA_LAUNCH_CHECK("delta_rule_prepare");
+  return 0;
+}
+
+extern "C" int ra_delta_rule_scan(const float* qkv, int ld, float* gates, const float* a_log, const float* dt_bias,
+                                  float* state, long slot_stride, const int* cu_tokens, const int* state_slots,
+                                  const int* fresh, int n_seqs, int n_tokens, int heads, int key_heads, int key_dim,
+                                  int value_dim, float* out, hipStream_t stream) {
+  RA_CHECK(n_seqs > 0 && n_tokens > 0 && heads > 0 && key_heads > 0 && heads % key_heads == 0,
+           "delta_rule_scan: %d requests, %d tokens, %d heads on %d key heads", n_seqs, n_tokens, heads, key_heads);
+  ScanGeom g;
+  RA_CHECK(scan_geom(1, key_dim, value_dim, &g), "delta_rule_scan: heads of %d x %d (keys up to 512)", key_dim, value_dim);
+  RA_CHECK(slot_stride >= (long)heads * g.waves * g.wave_floats, "delta_rule_scan: a state slot of %ld floats, need %ld",
+           slot_stride, (long)heads * g.waves * g.wave_floats);
+  RA_CHECK(heads <= 65535, "delta_rule_scan: %d heads in one launch", heads);
+  const long n = (long)n_tokens * 2 * heads;
+  delta_rule_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(gates, a_log, dt_bias, heads, n);
+  RA_LAUNCH_CHECK("delta_rule_gates");
+  const ScanLaunch L = scan_launch(g, n_seqs, heads);
+#define RA_DS(R, NPL)                                                                                          \
+  delta_rule_scan_kernel<R, NPL><<<L.grid, L.threads, 0, stream>>>(qkv, ld, gates, state, slot_stride, cu_tokens, \
+                                                                  state_slots, fresh, heads, key_heads, key_dim,   \
+                                                                  value_dim, g.waves, out)
+#define RA_DS_N(R)                               \
+  do {                                           \
+    if (g.NPL == 2) RA_DS(R, 2);                 \
+    else if (g.NPL == 4) RA_DS(R, 4);            \
+    else if (g.NPL == 8) RA_DS(R, 8);            \
+    else RA_DS(R, 16);                           \
+  } while (0)
+  if (g.R == 8) RA_DS_N(8); else RA_DS_N(32);
+#undef RA_DS_N
+#undef RA_DS
+  RA_LAUNCH_CHECK("delta_rule_scan");
+  return 0;
+}
+
+extern "C" int ra_head_norm_gate(const float* read, const float* weight, int per_head_weight, const void* gate,
+                                 int ldg, int act_dtype, int silu, float eps, int n_tokens, int heads, int value_dim,
+                                 void* out, hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && heads > 0 && value_dim > 0, "head_norm_gate: %d tokens, %d heads of %d", n_tokens, heads,
+           value_dim);
+  const long units = (long)n_tokens * heads;
+  const unsigned blocks = (unsigned)((units + 3) / 4);
+  const int ws = per_head_weight ? value_dim : 0;
+  if (act_dtype == RA_F32)
+    head_norm_gate_kernel<float><<<blocks, 4 * RA_WAVE, 0, stream>>>(read, weight, ws, (const float*)gate, ldg, silu,
+                                                                     eps, heads, value_dim, (float*)out, units);
+  else if (act_dtype == RA_BF16)
+    head_norm_gate_kernel<bf16_t><<<blocks, 4 * RA_WAVE, 0, stream>>>(read, weight, ws, (const bf16_t*)gate, ldg, silu,
+                                                                      eps, heads, value_dim, (bf16_t*)out, units);
+  else
+    return ra_fail("head_norm_gate: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("head_norm_gate");
+  return 0;
+}
+
+extern "C" int ra_normed_mean(const void* const* xs, const float* const* ws, int n, int act_dtype, float eps,
+                              int n_tokens, int hidden, void* out, float* resid, float scale, hipStream_t stream) {
+  RA_CHECK(n >= 1 && n <= MEAN_MAX, "normed_mean: %d inputs (1 to %d)", n, MEAN_MAX);
+  RA_CHECK(n_tokens > 0 && hidden > 0, "normed_mean: %d tokens, width %d", n_tokens, hidden);
+  RA_CHECK((out == nullptr) != (resid == nullptr), "normed_mean: the result goes into the stream or into out");
+  MeanInputs in;
+  for (int i = 0; i < MEAN_MAX; ++i) {
+    in.x[i] = i < n ? xs[i] : nullptr;
+    in.w[i] = i < n ? ws[i] : nullptr;
+  }
+  if (act_dtype == RA_F32)
+    normed_mean_kernel<float><<<n_tokens, 256, 0, stream>>>(in, n, eps, hidden, (float*)out, resid, scale);
+  else if (act_dtype == RA_BF16)
+    normed_mean_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(in, n, eps, hidden, (bf16_t*)out, resid, scale);
+  else
+    return ra_fail("normed_mean: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("normed_mean");
+  return 0;
+}

@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 19
+#define RA_ABI_VERSION 20
 
 #ifdef __cplusplus
 extern "C" {
@@ -15,10 +15,11 @@ const char* ra_last_error(void);
 int ra_abi_version(void);
 
 int ra_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens, int hidden,
-             hipStream_t stream);
+             float scale, hipStream_t stream);
 
 int ra_add_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype, void* out,
-                   int act_dtype, const int* rows, int n_rows, int hidden, float eps, hipStream_t stream);
+                   int act_dtype, const int* rows, int n_rows, int hidden, float eps, float delta_scale,
+                   hipStream_t stream);
 
 int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
                           int weight_dtype, float eps, const int* positions, const float* inv_freq,
@@ -175,7 +176,7 @@ int ra_pair_hash_add(float* resid, const void* table, int table_dtype, const int
                      hipStream_t stream);
 // resid[t, :] += delta[t, :] + other[t, :] + vec[:]; every addend may be null
 int ra_stream_add(float* resid, const void* delta, int delta_dtype, const float* other, const void* vec,
-                  int vec_dtype, int n_tokens, int hidden, hipStream_t stream);
+                  int vec_dtype, int n_tokens, int hidden, float delta_scale, hipStream_t stream);
 // logits <- cap * tanh(logits / cap) in place
 int ra_tanh_cap(float* logits, int n_rows, int vocab, int row_stride, float cap, hipStream_t stream);
 
@@ -209,6 +210,42 @@ int ra_moe_up_chosen(const void* x, int ldx, const void* w_up, const int* ids, c
                      int act_dtype, int n_tokens, int top, int experts, int ff, int width, hipStream_t stream);
 int ra_moe_down_chosen(const void* act, const void* w_down, const int* ids, float* resid, void* out, int act_dtype,
                        int n_tokens, int top, int experts, int ff, int width, hipStream_t stream);
+
+// sigmoid scores, groups of experts of which the best `kept` stay (a group's score: the sum of its `group_top`
+// largest), then the `top` largest; weights = score * scale, not renormalised
+int ra_moe_route_sigmoid(const float* logits, int ld, int experts, int top, int groups, int kept, int group_top,
+                         float scale, int* ids, float* weights, int n_tokens, hipStream_t stream);
+// gu [n_tokens, 2 (experts ff + shared)]: [gate | up] an expert, the shared expert's behind them;
+// act [n_tokens, experts ff + shared] = weight * silu(gate) * up (0 for experts not chosen, weight 1 for the shared one)
+int ra_moe_silu_gate_scale(const void* gu, void* act, int act_dtype, const int* ids, const float* weights, int top,
+                           int experts, int ff, int shared, int n_tokens, hipStream_t stream);
+
+// ---- recurrent mixers (recurrent.hip) ----
+// floats of state a request slot holds for the scan kernels; kind 0: matrix memory, 1: delta rule; -1: sizes not taken
+long ra_scan_state_floats(int kind, int heads, int key_dim, int value_dim);
+// gates [n_tokens, 2 heads] float pre-activations (input | forget), turned into log gates in place; proj rows hold
+// q, k (heads x key_dim) and v (heads x value_dim) at the given column offsets; out float [n_tokens, heads * value_dim]
+int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, int q_off, int k_off, int v_off, float* gates,
+                          const float* gate_bias, float* state, long slot_stride, const int* cu_tokens,
+                          const int* state_slots, const int* fresh, int n_seqs, int n_tokens, int heads, int key_dim,
+                          int value_dim, float gate_cap, float q_scale, float denom_eps, float* out,
+                          hipStream_t stream);
+// proj rows hold q | k (key_heads x key_dim each) | v (heads x value_dim) from column 0; filt float [channels, taps];
+// the filter's tail lies at tail_off floats in a request's state slot; qkv float [n_tokens, channels]
+int ra_delta_rule_prepare(const void* proj, int act_dtype, int ld, const float* filt, float* state, long slot_stride,
+                          long tail_off, const int* seq_of_token, const int* cu_tokens, const int* state_slots,
+                          const int* fresh, int n_seqs, int n_tokens, int key_heads, int key_dim, int heads,
+                          int value_dim, int taps, float unit_eps, float q_scale, float* qkv, hipStream_t stream);
+// gates [n_tokens, 2 heads] float pre-activations (b | a), turned into (beta | decay) in place
+int ra_delta_rule_scan(const float* qkv, int ld, float* gates, const float* a_log, const float* dt_bias, float* state,
+                       long slot_stride, const int* cu_tokens, const int* state_slots, const int* fresh, int n_seqs,
+                       int n_tokens, int heads, int key_heads, int key_dim, int value_dim, float* out,
+                       hipStream_t stream);
+int ra_head_norm_gate(const float* read, const float* weight, int per_head_weight, const void* gate, int ldg,
+                      int act_dtype, int silu, float eps, int n_tokens, int heads, int value_dim, void* out,
+                      hipStream_t stream);
+int ra_normed_mean(const void* const* xs, const float* const* ws, int n, int act_dtype, float eps, int n_tokens,
+                   int hidden, void* out, float* resid, float scale, hipStream_t stream);
 
 #ifdef __cplusplus
 }

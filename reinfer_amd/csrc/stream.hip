@@ -67,15 +67,16 @@ extern "C" int ra_pair_hash_add(float* resid, const void* table, int table_dtype
 }
 
 // ---------------------------------------------------------------------------
-// resid[t, :] += delta[t, :] + other[t, :] + vec[:]   (each addend optional)
+// resid[t, :] += delta_scale * delta[t, :] + other[t, :] + vec[:]   (each addend optional)
 // ---------------------------------------------------------------------------
 template <typename TD, typename TV>
 __global__ void stream_add_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
-                                  const float* __restrict__ other, const TV* __restrict__ vec, int h) {
+                                  const float* __restrict__ other, const TV* __restrict__ vec, int h,
+                                  float dscale) {
   const size_t base = (size_t)blockIdx.x * h;
   for (int i = threadIdx.x; i < h; i += blockDim.x) {
     float v = resid[base + i];
-    if (delta) v += to_f32(delta[base + i]);
+    if (delta) v += dscale * to_f32(delta[base + i]);
     if (other) v += other[base + i];
     if (vec) v += to_f32(vec[i]);
     resid[base + i] = v;
@@ -83,10 +84,10 @@ __global__ void stream_add_kernel(float* __restrict__ resid, const TD* __restric
 }
 
 extern "C" int ra_stream_add(float* resid, const void* delta, int delta_dtype, const float* other, const void* vec,
-                             int vec_dtype, int n_tokens, int hidden, hipStream_t stream) {
+                             int vec_dtype, int n_tokens, int hidden, float delta_scale, hipStream_t stream) {
   RA_CHECK(n_tokens > 0 && hidden > 0, "stream_add: empty input (%d tokens, width %d)", n_tokens, hidden);
 #define RA_SA(TD, TV)                                                                                    \
-  stream_add_kernel<TD, TV><<<n_tokens, 256, 0, stream>>>(resid, (const TD*)delta, other, (const TV*)vec, hidden)
+  stream_add_kernel<TD, TV><<<n_tokens, 256, 0, stream>>>(resid, (const TD*)delta, other, (const TV*)vec, hidden, delta_scale)
   if (delta_dtype == RA_F32 && vec_dtype == RA_F32) RA_SA(float, float);
   else if (delta_dtype == RA_F32 && vec_dtype == RA_BF16) RA_SA(float, bf16_t);
   else if (delta_dtype == RA_BF16 && vec_dtype == RA_F32) RA_SA(bf16_t, float);

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 
 class KernelLibraryError(RuntimeError):
@@ -29,8 +29,8 @@ _lib_path: Optional[str] = None
 P, I, F = c_void_p, c_int, c_float
 
 _SIGNATURES = {
-    "ra_embed": [P, I, P, P, I, I, P],
-    "ra_add_rmsnorm": [P, P, P, I, P, I, P, I, I, F, P],
+    "ra_embed": [P, I, P, P, I, I, F, P],
+    "ra_add_rmsnorm": [P, P, P, I, P, I, P, I, I, F, F, P],
     "ra_qk_norm_rope_cache": [P, I, P, P, I, F, P, P, I, I, P, P, P, I, I, I, I, I, P],
     "ra_qk_norm_rope_cache_sums": [P, I, P, I, F, I, P, I, I, P, P, I, F, P, P, I, I, P, P, P, I, I, I, I, I, P],
     "ra_gemm_wide_partial": [P, P, P, c_long, I, I, I, I, P],
@@ -48,7 +48,7 @@ _SIGNATURES = {
     "ra_sample_static": [P, I, I, I, P, P, P, P, P],
     "ra_filter_logits": [P, I, I, I, P, P, P],
     "ra_pair_hash_add": [P, P, I, P, P, P, P, P, P, I, c_longlong, c_longlong, I, I, P],
-    "ra_stream_add": [P, P, I, P, P, I, I, I, P],
+    "ra_stream_add": [P, P, I, P, P, I, I, I, F, P],
     "ra_tanh_cap": [P, I, I, I, F, P],
     "ra_latent_prep": [P, I, I, I, I, P, I, F, P, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
     "ra_head_linear": [P, I, I, P, P, I, I, P, I, I, I, I, I, I, P],
@@ -56,6 +56,13 @@ _SIGNATURES = {
     "ra_moe_relu2_scale": [P, P, I, P, P, I, I, I, I, P],
     "ra_moe_up_chosen": [P, I, P, P, P, P, I, I, I, I, I, I, P],
     "ra_moe_down_chosen": [P, P, P, P, P, I, I, I, I, I, I, P],
+    "ra_moe_route_sigmoid": [P, I, I, I, I, I, I, F, P, P, I, P],
+    "ra_moe_silu_gate_scale": [P, P, I, P, P, I, I, I, I, I, P],
+    "ra_matrix_memory_scan": [P, I, I, I, I, I, P, P, P, c_long, P, P, P, I, I, I, I, I, F, F, F, P, P],
+    "ra_delta_rule_prepare": [P, I, I, P, P, c_long, c_long, P, P, P, P, I, I, I, I, I, I, I, F, F, P, P],
+    "ra_delta_rule_scan": [P, I, P, P, P, P, c_long, P, P, P, I, I, I, I, I, I, P, P],
+    "ra_head_norm_gate": [P, P, I, P, I, I, I, F, I, I, I, P, P],
+    "ra_normed_mean": [P, P, I, I, F, I, I, P, P, F, P],
     "ra_stream_read": [P, c_long, P, P],
     "ra_mfma_loop": [I, I, I, P, P, P],
 }
@@ -95,6 +102,8 @@ def load() -> ctypes.CDLL:
         lib.ra_sample_static_max_pairs.argtypes = []
         lib.ra_sample_static_prepare.restype = c_int
         lib.ra_sample_static_prepare.argtypes = []
+        lib.ra_scan_state_floats.restype = c_long
+        lib.ra_scan_state_floats.argtypes = [c_int, c_int, c_int, c_int]
         lib.ra_gemm_skinny_max_rows.restype = c_int
         lib.ra_gemm_skinny_max_rows.argtypes = []
         lib.ra_gemm_skinny_row_parts.restype = c_int

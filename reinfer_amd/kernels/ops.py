@@ -59,7 +59,7 @@ class HipKernels:
         self._side_streams = {}     # device -> the stream for the second kernel of a mixed step
 
     # ------------------------------------------------------------------ rows
-    def embed(self, table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    def embed(self, table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
         _dev(table, ids, out)
         T, h = out.shape
         if table.dim() != 2 or table.shape[1] != h or not table.is_contiguous():
@@ -68,10 +68,11 @@ class HipKernels:
             raise TypeError("embed: the residual stream is contiguous float32")
         _int32(ids, "embed ids", T)
         library.call("ra_embed", table.data_ptr(), _tag(table, "embed table"), ids.data_ptr(),
-                     out.data_ptr(), T, h, _stream())
+                     out.data_ptr(), T, h, float(scale), _stream())
 
     def add_rmsnorm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
-                    eps: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+                    eps: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                    delta_scale: float = 1.0) -> None:
         _dev(resid, delta, weight, out, rows)
         h = resid.shape[-1]
         n = out.shape[0]
@@ -89,7 +90,7 @@ class HipKernels:
             _int32(rows, "add_rmsnorm rows", n)
         library.call("ra_add_rmsnorm", resid.data_ptr(), _ptr(delta), weight.data_ptr(),
                      _tag(weight, "norm weight"), out.data_ptr(), _tag(out, "add_rmsnorm out"),
-                     _ptr(rows), n, h, float(eps), _stream())
+                     _ptr(rows), n, h, float(eps), float(delta_scale), _stream())
 
     def qk_norm_rope_cache(self, qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
                            k_weight: Optional[torch.Tensor], eps: float, positions: torch.Tensor,
@@ -880,9 +881,10 @@ class HipKernels:
                      int(mul_prev), int(mul_cur), T, h, _stream())
 
     def stream_add(self, resid: torch.Tensor, delta: Optional[torch.Tensor] = None,
-                   other: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None) -> None:
-        """resid += delta + other + vec: ``delta`` [T, width] in either dtype, ``other`` [T, width] float32,
-        ``vec`` [width] in either dtype; each may be None."""
+                   other: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None,
+                   delta_scale: float = 1.0) -> None:
+        """resid += delta_scale * delta + other + vec: ``delta`` [T, width] in either dtype, ``other`` [T, width]
+        float32, ``vec`` [width] in either dtype; each may be None."""
         _dev(resid, delta, other, vec)
         T, h = resid.shape
         if resid.dtype != torch.float32 or not resid.is_contiguous():
@@ -896,7 +898,8 @@ class HipKernels:
         if delta is None and other is None and vec is None:
             return
         library.call("ra_stream_add", resid.data_ptr(), _ptr(delta), _tag(delta, "stream_add delta") if delta is not None else 0,
-                     _ptr(other), _ptr(vec), _tag(vec, "stream_add vector") if vec is not None else 0, T, h, _stream())
+                     _ptr(other), _ptr(vec), _tag(vec, "stream_add vector") if vec is not None else 0, T, h,
+                     float(delta_scale), _stream())
 
     def tanh_cap(self, logits: torch.Tensor, cap: float) -> None:
         """logits <- cap * tanh(logits / cap), in place."""
@@ -963,13 +966,161 @@ class HipKernels:
                      out.stride(0), int(o_head), _ptr(gate), gate.stride(0) if gate is not None else 0,
                      _tag(x, "head_linear"), T, H, N, K, _stream())
 
+    # ------------------------------------------------------ recurrent mixers
+    _SCAN_KINDS = {"matrix_memory": 0, "delta_rule": 1}
+
+    def scan_state_floats(self, kind: str, heads: int, key_dim: int, value_dim: int) -> int:
+        """Floats of a request's state slot that the scan kernel of ``kind`` ("matrix_memory", "delta_rule")
+        keeps for ``heads`` heads of [key_dim, value_dim], in the kernel's own layout."""
+        n = int(library.load().ra_scan_state_floats(self._SCAN_KINDS[kind], int(heads), int(key_dim), int(value_dim)))
+        if n < 0:
+            raise ValueError(f"{kind}: heads of {key_dim} x {value_dim} are not taken (keys up to 512)")
+        return n
+
+    @staticmethod
+    def _check_scan(what: str, state: torch.Tensor, batch, T: int) -> None:
+        if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous():
+            raise TypeError(f"{what}: the state is contiguous float32 [slots, floats]")
+        if T != batch.num_tokens:
+            raise ValueError(f"{what}: {T} rows for a step of {batch.num_tokens} tokens")
+        _int32(batch.cu_tokens, "first token of each request", batch.num_seqs + 1)
+        _int32(batch.state_slots, "state slots", batch.num_seqs)
+        _int32(batch.fresh, "first-step flags", batch.num_seqs)
+        _int32(batch.seq_of_token, "request of each token", T)
+
+    def matrix_memory_scan(self, proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: torch.Tensor,
+                           gate_bias: torch.Tensor, state: torch.Tensor, batch, heads: int, key_dim: int,
+                           value_dim: int, gate_cap: float, q_scale: float, denom_eps: float,
+                           out: torch.Tensor) -> None:
+        """The matrix memory over the step's tokens, request by request in order, from and into ``state``
+        [slots, floats]. ``proj`` [T, *] holds q and k (heads x key_dim) and v (heads x value_dim) from the
+        given columns; ``gates`` float32 [T, 2 heads] holds the input and forget gates' pre-activations and
+        is overwritten with the log gates; ``out`` float32 [T, heads * value_dim] gets the read-out before
+        its norm."""
+        _dev(proj, gates, gate_bias, state, out)
+        T = proj.shape[0]
+        self._check_scan("matrix_memory_scan", state, batch, T)
+        if proj.dim() != 2 or proj.stride(1) != 1 or max(q_off, k_off) + heads * key_dim > proj.shape[1] \
+                or v_off + heads * value_dim > proj.shape[1]:
+            raise ValueError(f"matrix_memory_scan: rows of {tuple(proj.shape)} do not hold q, k, v at {q_off}, {k_off}, {v_off}")
+        if gates.shape != (T, 2 * heads) or gates.dtype != torch.float32 or not gates.is_contiguous() \
+                or gate_bias.shape != (2 * heads,) or gate_bias.dtype != torch.float32 or not gate_bias.is_contiguous():
+            raise ValueError("matrix_memory_scan: gates float32 [T, 2 heads], their bias float32 [2 heads]")
+        if out.shape != (T, heads * value_dim) or out.dtype != torch.float32 or not out.is_contiguous():
+            raise ValueError("matrix_memory_scan: out is contiguous float32 [T, heads * value_dim]")
+        library.call("ra_matrix_memory_scan", proj.data_ptr(), _tag(proj, "matrix_memory_scan"), proj.stride(0),
+                     int(q_off), int(k_off), int(v_off), gates.data_ptr(), gate_bias.data_ptr(), state.data_ptr(),
+                     state.stride(0), batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), batch.fresh.data_ptr(),
+                     batch.num_seqs, T, int(heads), int(key_dim), int(value_dim), float(gate_cap), float(q_scale),
+                     float(denom_eps), out.data_ptr(), _stream())
+
+    def delta_rule_prepare(self, proj: torch.Tensor, filt: torch.Tensor, state: torch.Tensor, tail_off: int, batch,
+                           key_heads: int, key_dim: int, heads: int, value_dim: int, taps: int, unit_eps: float,
+                           q_scale: float, qkv: torch.Tensor) -> None:
+        """The delta rule's inputs: the causal filter over time (``filt`` float32 [channels, taps]; rows before
+        the step's portion come from the ``taps - 1`` rows kept at ``tail_off`` in the request's state, which
+        then move on), silu, unit norms of the q and k heads. ``proj`` [T, >= channels] holds q | k | v from
+        column 0; ``qkv`` float32 [T, channels] gets the results."""
+        _dev(proj, filt, state, qkv)
+        T = proj.shape[0]
+        C = 2 * key_heads * key_dim + heads * value_dim
+        self._check_scan("delta_rule_prepare", state, batch, T)
+        if proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < C:
+            raise ValueError(f"delta_rule_prepare: rows of {tuple(proj.shape)} do not hold {C} channels")
+        if filt.shape != (C, taps) or filt.dtype != torch.float32 or not filt.is_contiguous():
+            raise ValueError(f"delta_rule_prepare: filter {tuple(filt.shape)} {filt.dtype}, expected float32 [{C}, {taps}]")
+        if qkv.shape != (T, C) or qkv.dtype != torch.float32 or not qkv.is_contiguous():
+            raise ValueError(f"delta_rule_prepare: qkv is contiguous float32 [T, {C}]")
+        if state.shape[1] < tail_off + (taps - 1) * C:
+            raise ValueError("delta_rule_prepare: the state slot does not hold the filter's tail")
+        library.call("ra_delta_rule_prepare", proj.data_ptr(), _tag(proj, "delta_rule_prepare"), proj.stride(0),
+                     filt.data_ptr(), state.data_ptr(), state.stride(0), int(tail_off), batch.seq_of_token.data_ptr(),
+                     batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), batch.fresh.data_ptr(), batch.num_seqs,
+                     T, int(key_heads), int(key_dim), int(heads), int(value_dim), int(taps), float(unit_eps),
+                     float(q_scale), qkv.data_ptr(), _stream())
+
+    def delta_rule_scan(self, qkv: torch.Tensor, gates: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                        state: torch.Tensor, batch, heads: int, key_heads: int, key_dim: int, value_dim: int,
+                        out: torch.Tensor) -> None:
+        """The gated delta rule over the step's tokens from and into ``state``. ``qkv`` float32 [T, q | k | v]
+        as ``delta_rule_prepare`` left it; ``gates`` float32 [T, 2 heads] holds the pre-activations of beta
+        and of the decay and is overwritten with both; ``out`` float32 [T, heads * value_dim]."""
+        _dev(qkv, gates, a_log, dt_bias, state, out)
+        T = qkv.shape[0]
+        C = 2 * key_heads * key_dim + heads * value_dim
+        self._check_scan("delta_rule_scan", state, batch, T)
+        if qkv.shape != (T, C) or qkv.dtype != torch.float32 or not qkv.is_contiguous():
+            raise ValueError(f"delta_rule_scan: qkv is contiguous float32 [T, {C}]")
+        if gates.shape != (T, 2 * heads) or gates.dtype != torch.float32 or not gates.is_contiguous():
+            raise ValueError("delta_rule_scan: gates float32 [T, 2 heads]")
+        for v, what in ((a_log, "A_log"), (dt_bias, "dt_bias")):
+            if v.shape != (heads,) or v.dtype != torch.float32 or not v.is_contiguous():
+                raise ValueError(f"delta_rule_scan: {what} is float32 [heads]")
+        if out.shape != (T, heads * value_dim) or out.dtype != torch.float32 or not out.is_contiguous():
+            raise ValueError("delta_rule_scan: out is contiguous float32 [T, heads * value_dim]")
+        library.call("ra_delta_rule_scan", qkv.data_ptr(), qkv.stride(0), gates.data_ptr(), a_log.data_ptr(),
+                     dt_bias.data_ptr(), state.data_ptr(), state.stride(0), batch.cu_tokens.data_ptr(),
+                     batch.state_slots.data_ptr(), batch.fresh.data_ptr(), batch.num_seqs, T, int(heads),
+                     int(key_heads), int(key_dim), int(value_dim), out.data_ptr(), _stream())
+
+    def head_norm_gate(self, read: torch.Tensor, weight: torch.Tensor, per_head: bool, gate: torch.Tensor, kind: str,
+                       eps: float, heads: int, value_dim: int, out: torch.Tensor) -> None:
+        """out[t, h] = read[t, h] / rms(read[t, h]) * weight * act(gate[t, h]) head by head: ``read`` float32
+        [T, heads * value_dim], ``weight`` float32 [heads * value_dim] (``per_head``) or [value_dim] for all
+        heads, ``gate`` [T, >= heads * value_dim] rows of the activations' dtype, ``kind`` "sigmoid" or "silu"."""
+        _dev(read, weight, gate, out)
+        T = read.shape[0]
+        n = heads * value_dim
+        if read.shape != (T, n) or read.dtype != torch.float32 or not read.is_contiguous():
+            raise ValueError(f"head_norm_gate: read is contiguous float32 [T, {n}]")
+        if weight.dtype != torch.float32 or weight.shape != ((n,) if per_head else (value_dim,)) or not weight.is_contiguous():
+            raise ValueError(f"head_norm_gate: weight {tuple(weight.shape)} {weight.dtype}")
+        if gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < n or gate.stride(1) != 1 or gate.dtype != out.dtype:
+            raise ValueError(f"head_norm_gate: gate {tuple(gate.shape)}, expected rows of at least {n} in the output's dtype")
+        if out.shape != (T, n) or not out.is_contiguous():
+            raise ValueError(f"head_norm_gate: out is contiguous [T, {n}]")
+        if kind not in ("sigmoid", "silu"):
+            raise ValueError(f"head_norm_gate: gate kind {kind!r}")
+        library.call("ra_head_norm_gate", read.data_ptr(), weight.data_ptr(), 1 if per_head else 0, gate.data_ptr(),
+                     gate.stride(0), _tag(out, "head_norm_gate"), 1 if kind == "silu" else 0, float(eps), T, int(heads),
+                     int(value_dim), out.data_ptr(), _stream())
+
+    def normed_mean(self, xs, weights, eps: float, out: Optional[torch.Tensor] = None,
+                    resid: Optional[torch.Tensor] = None, scale: float = 1.0) -> None:
+        """y = mean_i xs[i] / rms(xs[i]) * weights[i] row by row (float); written to ``out`` (the inputs' dtype)
+        or ``resid += scale * y`` (the float stream): exactly one of the two is given."""
+        import ctypes
+        n = len(xs)
+        if not 1 <= n <= 4 or len(weights) != n:
+            raise ValueError(f"normed_mean: {n} inputs with {len(weights)} weights (1 to 4 of each)")
+        _dev(*xs, *weights, out, resid)
+        T, h = xs[0].shape
+        for x, w in zip(xs, weights):
+            if x.shape != (T, h) or x.dtype != xs[0].dtype or not x.is_contiguous():
+                raise ValueError("normed_mean: the inputs are contiguous [T, width] of one dtype")
+            if w.shape != (h,) or w.dtype != torch.float32 or not w.is_contiguous():
+                raise ValueError(f"normed_mean: weights are float32 [{h}]")
+        if (out is None) == (resid is None):
+            raise ValueError("normed_mean: the result goes into the stream or into out")
+        if out is not None and (out.shape != (T, h) or out.dtype != xs[0].dtype or not out.is_contiguous()):
+            raise ValueError("normed_mean: out is contiguous [T, width] in the inputs' dtype")
+        if resid is not None and (resid.shape != (T, h) or resid.dtype != torch.float32 or not resid.is_contiguous()):
+            raise ValueError("normed_mean: the residual stream is contiguous float32 [T, width]")
+        px = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+        pw = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
+        library.call("ra_normed_mean", px, pw, n, _tag(xs[0], "normed_mean"), float(eps), T, h, _ptr(out), _ptr(resid),
+                     float(scale), _stream())
+
     # ---------------------------------------------------- mixture of experts
     def moe_route(self, x: torch.Tensor, router: torch.Tensor, top: int, ids: torch.Tensor,
-                  weights: torch.Tensor) -> None:
+                  weights: torch.Tensor, scoring: str = "softmax_chosen", scale: float = 1.0, groups: int = 1,
+                  groups_kept: int = 1, group_top: int = 2) -> None:
         """Router logits x . router^T accumulated and kept in float (``router`` [experts, width] in the
         activations' dtype: a bfloat16 product's terms are exact in float), the ``top`` largest a token in
         falling order into ``ids`` [T, top] (int32), the softmax over those alone into ``weights`` [T, top]
-        (float32)."""
+        (float32). ``scoring`` "sigmoid": scores are the logits' sigmoids; with ``groups`` > 1 only experts of
+        the ``groups_kept`` best groups of neighbours (a group's score: the sum of its ``group_top`` largest
+        scores) can be chosen; the weights are the chosen scores times ``scale``."""
         _dev(x, router, ids, weights)
         T, width = x.shape
         E = router.shape[0]
@@ -981,8 +1132,31 @@ class HipKernels:
             raise ValueError(f"moe_route: ids int32 and weights float32, both [{T}, {top}]")
         logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
         self.linear(x, router, logits)
+        if scoring == "sigmoid":
+            library.call("ra_moe_route_sigmoid", logits.data_ptr(), logits.stride(0), E, int(top), int(groups),
+                         int(groups_kept), int(group_top), float(scale), ids.data_ptr(), weights.data_ptr(), T,
+                         _stream())
+            return
+        if scoring != "softmax_chosen":
+            raise ValueError(f"moe_route: scoring {scoring!r}")
         library.call("ra_moe_topk", logits.data_ptr(), logits.stride(0), E, int(top), ids.data_ptr(),
                      weights.data_ptr(), T, _stream())
+
+    def moe_silu_gate_scale(self, gu: torch.Tensor, act: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+                            experts: int, ff: int, shared: int = 0) -> None:
+        """``gu`` [T, 2 (experts ff + shared)]: [gate | up] of each expert, a shared expert's behind them.
+        act[t, e ff + j] = weight(t, e) silu(gate) up for the chosen experts, 0 for the others; the shared
+        expert's columns behind them with weight 1."""
+        _dev(gu, act, ids, weights)
+        T = gu.shape[0]
+        n = experts * ff + shared
+        if gu.shape != (T, 2 * n) or act.shape != (T, n) or act.dtype != gu.dtype or not gu.is_contiguous() \
+                or not act.is_contiguous():
+            raise ValueError(f"moe_silu_gate_scale: gu {tuple(gu.shape)} / act {tuple(act.shape)}, expected "
+                             f"[T, {2 * n}] and [T, {n}]")
+        self._check_choice("moe_silu_gate_scale", ids, weights, T, ids.shape[1])
+        library.call("ra_moe_silu_gate_scale", gu.data_ptr(), act.data_ptr(), _tag(gu, "moe_silu_gate_scale"),
+                     ids.data_ptr(), weights.data_ptr(), ids.shape[1], int(experts), int(ff), int(shared), T, _stream())
 
     def moe_relu2_scale(self, up: torch.Tensor, act: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
                         experts: int, ff: int) -> None:
