@@ -79,20 +79,22 @@ __global__ void moe_route_sigmoid_kernel(const float* __restrict__ logits, int l
   __builtin_amdgcn_wave_barrier();
   if (groups > 1) {
     const int size = E / groups;
-    // a lane scores whole groups: the sum of the group's `group_top` largest, found by striking in a private copy
+    // a lane scores whole groups: the sum of the group's `group_top` largest, each round taking the largest that
+    // comes behind the round before's in the order (score falling, index rising)
     for (int g = lane; g < groups; g += RA_WAVE) {
-      float sum = 0.f;
-      unsigned long long taken = 0ull;       // groups of up to 64 experts mark their taken ones here
+      float sum = 0.f, prev = INFINITY;
+      int prev_at = -1;
       for (int r = 0; r < group_top && r < size; ++r) {
         float best = -INFINITY;
         int at = -1;
         for (int i = 0; i < size; ++i) {
-          if (size <= 64 && ((taken >> i) & 1ull)) continue;
           const float v = s[g * size + i];
-          if (v > best) { best = v; at = i; }
+          const bool behind = v < prev || (v == prev && i > prev_at);
+          if (behind && (at < 0 || v > best)) { best = v; at = i; }
         }
         sum += best;
-        if (size <= 64) taken |= 1ull << at;
+        prev = best;
+        prev_at = at;
       }
       gs[g] = sum;
     }
@@ -149,8 +151,6 @@ extern "C" int ra_moe_route_sigmoid(const float* logits, int ld, int experts, in
   RA_CHECK(n_tokens > 0 && experts > 0, "moe_route_sigmoid: %d tokens, %d experts", n_tokens, experts);
   RA_CHECK(groups >= 1 && experts % groups == 0 && kept >= 1 && kept <= groups && group_top >= 1,
            "moe_route_sigmoid: %d experts in %d groups, %d kept, scored by %d", experts, groups, kept, group_top);
-  RA_CHECK(groups == 1 || experts / groups <= 64 || group_top == 1,
-           "moe_route_sigmoid: groups of %d experts (up to 64)", experts / groups);
   RA_CHECK(top > 0 && top <= RA_WAVE && top <= kept * (experts / groups),
            "moe_route_sigmoid: %d of %d experts that can be chosen (at most 64)", top, kept * (experts / groups));
   RA_CHECK(ld >= experts, "moe_route_sigmoid: rows of %d for %d experts", ld, experts);
