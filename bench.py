@@ -389,8 +389,46 @@ def design_sizes():
     return out
 
 
+# ---------------------------------------------------------------------------------------------------
+# --design kobolix: the Kobolix design beside the Qwen3 dense decoder at equal size
+# ---------------------------------------------------------------------------------------------------
+def _kobolix_raw(width, vocab, pattern, repeats, mem, attn, delta, dense_ff, moe):
+    """``pattern``: a string of layer codes, repeated: M matrix memory + dense, m matrix memory + experts,
+    P side-by-side + experts, p side-by-side + dense."""
+    memory = {"dim": mem[1], "gate_cap": 15.0, "heads": mem[0], "vdim": mem[2]}
+    pair = {"left": {"dim": attn[2], "heads": attn[0], "kv_heads": attn[1], "rot": {"base": 1000000.0, "dims": attn[2] // 2},
+                     "scale": attn[2] ** -0.5, "vdim": attn[3]},
+            "right": {"conv": 4, "dim": delta[2], "heads": delta[0], "kv_heads": delta[1], "vdim": delta[3]}}
+    dense = {"ff": dense_ff, "kind": "dense"}
+    experts = {"expert": {"ff": moe[2]}, "kind": "moe", "shared": {"ff": moe[3]},
+               "router": {"experts": moe[0], "groups": {"count": 4, "keep": 2}, "scale": 2.5, "top": moe[1]}}
+    kinds = {"M": ("mlstm", memory, dense), "m": ("mlstm", memory, experts), "P": ("parallel", pair, experts),
+             "p": ("parallel", pair, dense)}
+    layers = [{"type": kinds[c][0], "mixer": kinds[c][1], "mlp": kinds[c][2]} for c in pattern * repeats]
+    return {"architecture": "Kobolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "embedding": {"scale": 8.0}, "layers": layers}
+
+
+# (name, Kobolix configuration, its Qwen3 twin): as many layers, the same width and attention heads, a dense
+# feed-forward with the parameters of a token's chosen experts and the shared one
+def kobolix_sizes():
+    out = []
+    for name, width, repeats, mem, attn, delta, dense_ff, moe in (
+            ("w2048", 2048, 2, (8, 128, 256), (16, 4, 128, 128), (16, 8, 128, 128), 5632, (16, 4, 512, 1024)),
+            ("w4096", 4096, 2, (16, 128, 256), (32, 8, 128, 128), (32, 16, 128, 128), 11008, (16, 4, 1024, 2048))):
+        vocab = 32768
+        pattern = "MPm"
+        twin = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "num_hidden_layers": len(pattern) * repeats,
+                "hidden_size": width, "num_attention_heads": attn[0], "num_key_value_heads": attn[1], "head_dim": 128,
+                "intermediate_size": moe[1] * moe[2] + moe[3], "vocab_size": vocab, "rope_theta": 1000000.0,
+                "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 8192,
+                "attention_bias": False}
+        out.append((name, _kobolix_raw(width, vocab, pattern, repeats, mem, attn, delta, dense_ff, moe), twin, vocab))
+    return out
+
+
 def design_run(args) -> int:
-    """Prefill and decode throughput of Puresun and of its Qwen3 twin at each size, and the GPU time of a
+    """Prefill and decode throughput of the design (``--design``) and of its Qwen3 twin at each size, and the GPU time of a
     2,048-token prompt step and of a decode step at batch 8 by kernel class with each class's share of its
     roofline (weight bytes over 8 TB/s or flops over 2.5 PFLOP/s, whichever is longer). One JSON line."""
     import gc
@@ -431,8 +469,8 @@ def design_run(args) -> int:
         return out
 
     results = {}
-    for name, p_raw, q_raw, vocab in design_sizes():
-        for which, raw in (("puresun", p_raw), ("qwen3", q_raw)):
+    for name, p_raw, q_raw, vocab in (kobolix_sizes() if args.design == "kobolix" else design_sizes()):
+        for which, raw in ((args.design, p_raw), ("qwen3", q_raw)):
             cfg = config_from_dict(raw)
             log(f"{name} {which}: building ...")
             engine = LLMEngine(config=cfg, seed=args.seed, dtype=args.dtype, block_size=16,
@@ -460,7 +498,7 @@ def design_run(args) -> int:
             del engine
             gc.collect()
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "puresun_beside_qwen3", "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+    print(json.dumps({"metric": f"{args.design}_beside_qwen3", "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                       "data": "synthetic", "n_gpus": 1, "sizes": results}), flush=True)
     return 0
 
@@ -485,7 +523,7 @@ def main() -> int:
     ap.add_argument("--max-model-len", type=int, default=None, metavar="N",
                     help="context length (default: the shape's: 4096 at 8b, 8192 at 4b, 16384 at 32b)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the Qwen3-8B shape)")
-    ap.add_argument("--design", default=None, choices=["puresun"],
+    ap.add_argument("--design", default=None, choices=["puresun", "kobolix"],
                     help="instead of the default measurement: this design beside the Qwen3 decoder at equal sizes")
     args = ap.parse_args()
     if args.gpus != 1:

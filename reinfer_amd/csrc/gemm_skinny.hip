@@ -50,6 +50,7 @@ struct SkinnyNorm {
   bf16_t* out_x;           // [M, out_ldx] bf16(C_new * out_w)
   int out_ldx;
   float* out_ss;           // [workgroups, M] sums of squares of C_new over the workgroup's columns
+  float acc_scale;         // the accumulating epilogue adds acc_scale times the product (1: the product itself)
 };
 
 // What follows the walk over K in both kernels below: the waves' partial sums added in a fixed order,
@@ -145,7 +146,7 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], const floa
           if (m >= M || n >= N) continue;
           float v = acc[nt][mt][i];
           if (bias) v += to_f32(bias[n]);
-          v += pre.have_c ? pre.c[nt][mt][i] : to_f32(C[(size_t)m * ldc + n]);           // this thread alone owns (m, n)
+          v = v * nf.acc_scale + (pre.have_c ? pre.c[nt][mt][i] : to_f32(C[(size_t)m * ldc + n]));   // this thread alone owns (m, n)
           C[(size_t)m * ldc + n] = from_f32<TO>(v);
           const float w = pre.have_w ? __uint_as_float(nf.out_w_f32 ? pre.w[nt][i] : pre.w[nt][i] << 16)
                                      : (nf.out_w_f32 ? ((const float*)nf.out_w)[n] : to_f32(((const bf16_t*)nf.out_w)[n]));
@@ -172,7 +173,7 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], const floa
           float v = acc[nt][mt][i];
           if (bias) v += to_f32(bias[n]);
           const float c0 = pre.have_c ? pre.c[nt][mt][i] : to_f32(C[(size_t)m * ldc + n]);
-          C[(size_t)m * ldc + n] = from_f32<TO>(c0 + v);   // this thread alone owns (m, n)
+          C[(size_t)m * ldc + n] = from_f32<TO>(c0 + v * nf.acc_scale);   // this thread alone owns (m, n)
         }
       } else if (EPI == EPI_PLAIN) {
         if (m >= M) continue;
@@ -639,11 +640,11 @@ extern "C" int ra_gemm_skinny_row_parts(int M, int N) {
   return (N + f - 1) / f;
 }
 
-extern "C" int ra_gemm_skinny_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype,
-                                     int epilogue, int M, int N, int K, int lda, int ldc, const float* in_ss,
-                                     int in_parts, float in_eps, int in_width, const void* out_w,
-                                     int out_w_dtype, void* out_x, int out_ldx, float* out_ss,
-                                     hipStream_t stream) {
+static int gemm_skinny_impl(const void* A, const void* W, const void* bias, void* C, int out_dtype,
+                            int epilogue, int M, int N, int K, int lda, int ldc, const float* in_ss,
+                            int in_parts, float in_eps, int in_width, const void* out_w,
+                            int out_w_dtype, void* out_x, int out_ldx, float* out_ss, float acc_scale,
+                            hipStream_t stream) {
   RA_CHECK(M > 0 && N > 0 && K > 0, "gemm_skinny: empty product (%d, %d, %d)", M, N, K);
   RA_CHECK(M <= 64, "gemm_skinny: %d rows; this kernel takes at most 64", M);
   RA_CHECK(K % 8 == 0 && lda % 8 == 0, "gemm_skinny: K (%d) and the row stride (%d) must be multiples of 8", K, lda);
@@ -656,6 +657,7 @@ extern "C" int ra_gemm_skinny_normed(const void* A, const void* W, const void* b
   RA_CHECK(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_skinny: operands must be 16-byte aligned");
   RA_CHECK(out_dtype == RA_BF16 || out_dtype == RA_F32, "gemm_skinny: unknown output dtype tag %d", out_dtype);
   SkinnyNorm nf = {};
+  nf.acc_scale = acc_scale;
   if (in_ss) {
     RA_CHECK(in_parts > 0 && in_width > 0 && in_eps >= 0.f, "gemm_skinny: row sums need parts (%d), width (%d) and eps", in_parts, in_width);
     nf.in_ss = in_ss;
@@ -696,8 +698,24 @@ extern "C" int ra_gemm_skinny_normed(const void* A, const void* W, const void* b
   return launch_skinny<4, 2, 8, 2>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, nf, stream);
 }
 
+extern "C" int ra_gemm_skinny_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype,
+                                     int epilogue, int M, int N, int K, int lda, int ldc, const float* in_ss,
+                                     int in_parts, float in_eps, int in_width, const void* out_w,
+                                     int out_w_dtype, void* out_x, int out_ldx, float* out_ss,
+                                     hipStream_t stream) {
+  return gemm_skinny_impl(A, W, bias, C, out_dtype, epilogue, M, N, K, lda, ldc, in_ss, in_parts, in_eps, in_width,
+                          out_w, out_w_dtype, out_x, out_ldx, out_ss, 1.f, stream);
+}
+
 extern "C" int ra_gemm_skinny(const void* A, const void* W, const void* bias, void* C, int out_dtype,
                               int epilogue, int M, int N, int K, int lda, int ldc, hipStream_t stream) {
-  return ra_gemm_skinny_normed(A, W, bias, C, out_dtype, epilogue, M, N, K, lda, ldc, nullptr, 0, 0.f, 0, nullptr,
-                               0, nullptr, 0, nullptr, stream);
+  return gemm_skinny_impl(A, W, bias, C, out_dtype, epilogue, M, N, K, lda, ldc, nullptr, 0, 0.f, 0, nullptr,
+                          0, nullptr, 0, nullptr, 1.f, stream);
+}
+
+// C += acc_scale * (A . W^T): the accumulating epilogue with a factor on the product
+extern "C" int ra_gemm_skinny_scaled(const void* A, const void* W, float* C, int M, int N, int K, int lda, int ldc,
+                                     float acc_scale, hipStream_t stream) {
+  return gemm_skinny_impl(A, W, nullptr, C, RA_F32, EPI_ACCUM, M, N, K, lda, ldc, nullptr, 0, 0.f, 0, nullptr,
+                          0, nullptr, 0, nullptr, acc_scale, stream);
 }

@@ -40,6 +40,7 @@ struct WideNorm {
   int out_ldx;
   float* out_ss;           // [ceil(N / 1024), M] sums of squares of C_new over 1024 columns
   float out_eps;           // >= 0 with out_ss null: the adding kernel finishes the norm, out_x = bf16(norm(C_new) * out_w)
+  float acc_scale;         // the accumulating epilogue adds acc_scale times the product (1: the product itself)
 };
 
 #define GW_KS 128                      // k elements of a run
@@ -253,7 +254,7 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
         if (n >= N) continue;
         float v = acc[mt][i];
         if (bias) v += to_f32(bias[n]);
-        if (EPI == WEPI_ACCUM) v += to_f32(C[(size_t)m * ldc + n]);      // this thread alone owns (m, n)
+        if (EPI == WEPI_ACCUM) v = v * nf.acc_scale + to_f32(C[(size_t)m * ldc + n]);      // this thread alone owns (m, n)
         C[(size_t)m * ldc + n] = from_f32<TO>(v);
       }
     } else {
@@ -322,7 +323,7 @@ gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __rest
     if (n + i >= N) continue;
     float x = v[i] * rstd;
     if (bias) x += to_f32(bias[n + i]);
-    if (EPI == WEPI_ACCUM) x += to_f32(C[(size_t)m * ldc + n + i]);
+    if (EPI == WEPI_ACCUM) x = x * nf.acc_scale + to_f32(C[(size_t)m * ldc + n + i]);
     C[(size_t)m * ldc + n + i] = from_f32<TO>(x);
     if (EPI == WEPI_ACCUM && nf.out_x) {
       const float w = nf.out_w_f32 ? ((const float*)nf.out_w)[n + i] : to_f32(((const bf16_t*)nf.out_w)[n + i]);
@@ -379,7 +380,7 @@ gemm_wide_reduce_rows_kernel(const float* __restrict__ P, int S, const bf16_t* _
     for (int i = 0; i < 4; ++i) {
       float y = v[i] * rstd;
       if (bias) y += to_f32(bias[n + i]);
-      y += c0[i];
+      y = y * nf.acc_scale + c0[i];
       o[i] = y;
       x[c][i] = y;
       ss += y * y;
@@ -559,11 +560,11 @@ static int launch_wide(const void* A, int lda, const void* W, const void* bias, 
   return 0;
 }
 
-extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype,
-                                   int epilogue, int M, int N, int K, int lda, int ldc, float* scratch,
-                                   long scratch_floats, const float* in_ss, int in_parts, float in_eps,
-                                   int in_width, const void* out_w, int out_w_dtype, void* out_x, int out_ldx,
-                                   float* out_ss, float out_eps, hipStream_t stream) {
+static int gemm_wide_impl(const void* A, const void* W, const void* bias, void* C, int out_dtype,
+                          int epilogue, int M, int N, int K, int lda, int ldc, float* scratch,
+                          long scratch_floats, const float* in_ss, int in_parts, float in_eps,
+                          int in_width, const void* out_w, int out_w_dtype, void* out_x, int out_ldx,
+                          float* out_ss, float out_eps, float acc_scale, hipStream_t stream) {
   RA_CHECK(M > 0 && N > 0 && K > 0, "gemm_wide: empty product (%d, %d, %d)", M, N, K);
   RA_CHECK(M <= 128, "gemm_wide: %d rows; this kernel takes at most 128", M);
   RA_CHECK(K % 8 == 0 && lda % 8 == 0, "gemm_wide: K (%d) and the row stride (%d) must be multiples of 8", K, lda);
@@ -577,6 +578,7 @@ extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bia
   RA_CHECK(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_wide: operands must be 16-byte aligned");
   RA_CHECK(out_dtype == RA_BF16 || out_dtype == RA_F32, "gemm_wide: unknown output dtype tag %d", out_dtype);
   WideNorm nf = {};
+  nf.acc_scale = acc_scale;
   if (in_ss) {
     RA_CHECK(in_parts > 0 && in_width > 0 && in_eps >= 0.f, "gemm_wide: row sums need parts (%d), width (%d) and eps", in_parts, in_width);
     nf.in_ss = in_ss;
@@ -647,7 +649,8 @@ extern "C" int ra_gemm_wide_partial(const void* A, const void* W, float* P, long
   gw_split(WEPI_PLAIN, M, N, K, &waves, &S, &kps, &partial, true);
   RA_CHECK(P && p_floats >= (long)S * M * N, "gemm_wide: %d ranges of [%d, %d] need %ld floats, got %ld", S, M, N,
            (long)S * M * N, p_floats);
-  const WideNorm nf = {};
+  WideNorm nf = {};
+  nf.acc_scale = 1.f;
 #define RA_GWP(MT, WV)                                                                                  \
   gemm_wide_kernel<MT, WV, WEPI_PARTIAL, float><<<dim3((N + WV * 16 - 1) / (WV * 16), S), WV * RA_WAVE, 0, stream>>>( \
       (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, P, N, M, N, K, kps, nf)
@@ -662,9 +665,25 @@ extern "C" int ra_gemm_wide_partial(const void* A, const void* W, float* P, long
   return 0;
 }
 
+extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype,
+                                   int epilogue, int M, int N, int K, int lda, int ldc, float* scratch,
+                                   long scratch_floats, const float* in_ss, int in_parts, float in_eps,
+                                   int in_width, const void* out_w, int out_w_dtype, void* out_x, int out_ldx,
+                                   float* out_ss, float out_eps, hipStream_t stream) {
+  return gemm_wide_impl(A, W, bias, C, out_dtype, epilogue, M, N, K, lda, ldc, scratch, scratch_floats, in_ss,
+                        in_parts, in_eps, in_width, out_w, out_w_dtype, out_x, out_ldx, out_ss, out_eps, 1.f, stream);
+}
+
 extern "C" int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
                             int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
                             hipStream_t stream) {
-  return ra_gemm_wide_normed(A, W, bias, C, out_dtype, epilogue, M, N, K, lda, ldc, scratch, scratch_floats,
-                             nullptr, 0, 0.f, 0, nullptr, 0, nullptr, 0, nullptr, -1.f, stream);
+  return gemm_wide_impl(A, W, bias, C, out_dtype, epilogue, M, N, K, lda, ldc, scratch, scratch_floats,
+                        nullptr, 0, 0.f, 0, nullptr, 0, nullptr, 0, nullptr, -1.f, 1.f, stream);
+}
+
+// C += acc_scale * (A . W^T): the accumulating epilogue with a factor on the product
+extern "C" int ra_gemm_wide_scaled(const void* A, const void* W, float* C, int M, int N, int K, int lda, int ldc,
+                                   float* scratch, long scratch_floats, float acc_scale, hipStream_t stream) {
+  return gemm_wide_impl(A, W, nullptr, C, RA_F32, WEPI_ACCUM, M, N, K, lda, ldc, scratch, scratch_floats,
+                        nullptr, 0, 0.f, 0, nullptr, 0, nullptr, 0, nullptr, -1.f, acc_scale, stream);
 }

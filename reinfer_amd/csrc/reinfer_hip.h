@@ -220,6 +220,13 @@ int ra_moe_route_sigmoid(const float* logits, int ld, int experts, int top, int 
 int ra_moe_silu_gate_scale(const void* gu, void* act, int act_dtype, const int* ids, const float* weights, int top,
                            int experts, int ff, int shared, int n_tokens, hipStream_t stream);
 
+// C += acc_scale * (A . W^T) through the weight-streaming kernels (bfloat16 operands, float C; the limits of
+// ra_gemm_skinny / ra_gemm_wide with the accumulating epilogue)
+int ra_gemm_skinny_scaled(const void* A, const void* W, float* C, int M, int N, int K, int lda, int ldc,
+                          float acc_scale, hipStream_t stream);
+int ra_gemm_wide_scaled(const void* A, const void* W, float* C, int M, int N, int K, int lda, int ldc, float* scratch,
+                        long scratch_floats, float acc_scale, hipStream_t stream);
+
 // ---- recurrent mixers (recurrent.hip) ----
 // floats of state a request slot holds for the scan kernels; kind 0: matrix memory, 1: delta rule; -1: sizes not taken
 long ra_scan_state_floats(int kind, int heads, int key_dim, int value_dim);

@@ -43,6 +43,8 @@ _SIGNATURES = {
     "ra_gemm_wide": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P],
     "ra_gemm_wide_normed": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P, I, F, I, P, I, P, I, P, F, P],
     "ra_gemm_skinny_normed": [P, P, P, P, I, I, I, I, I, I, I, P, I, F, I, P, I, P, I, P, P],
+    "ra_gemm_skinny_scaled": [P, P, P, I, I, I, I, I, F, P],
+    "ra_gemm_wide_scaled": [P, P, P, I, I, I, I, I, P, c_long, F, P],
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],
     "ra_sample_static": [P, I, I, I, P, P, P, P, P],

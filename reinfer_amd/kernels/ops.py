@@ -659,7 +659,7 @@ class HipKernels:
                      out.stride(0), _stream())
 
     def linear_skinny(self, x, weight, out, bias=None, accumulate: bool = False, row_sums=None,
-                      emit=None, wide: Optional[bool] = None, finish=None):
+                      emit=None, wide: Optional[bool] = None, finish=None, alpha: float = 1.0):
         """The weight-streaming product; with ``accumulate`` the float32 ``out`` is added to (with more rows
         than the weight-streaming kernels take, by the library's product).
 
@@ -671,8 +671,28 @@ class HipKernels:
         rows of ss_out, as many as the kernel that ran has workgroups a row; that number comes back.
         ``finish`` = (w [N], x_out bfloat16 [M, N], eps), with ``accumulate`` and 65 to 128 rows, asks for the
         finished norm of the new ``out`` instead, x_out = bf16(rmsnorm(out, eps) * w): True comes back where
-        the product that ran wrote it (``can_finish_norm``), False where it only added."""
+        the product that ran wrote it (``can_finish_norm``), False where it only added.
+        ``alpha`` (with ``accumulate`` alone): out += alpha * (x . W^T)."""
         M, N, K = self._check_linear(x, weight, out, bias)
+        if alpha != 1.0:
+            if not accumulate or bias is not None or row_sums is not None or emit is not None or finish is not None \
+                    or x.dtype != torch.bfloat16 or out.dtype != torch.float32:
+                raise ValueError("linear_skinny: a factor rides on a plain accumulating bfloat16 product only")
+            lib = library.load()
+            if M > 64 and not bool(lib.ra_gemm_wide_preferred(2, M, N, K)):
+                torch.addmm(out, x, weight.t(), alpha=float(alpha), out_dtype=torch.float32, out=out)
+                return None
+            if wide is None:
+                wide = bool(lib.ra_gemm_wide_preferred(2, M, N, K))
+            if not wide:
+                library.call("ra_gemm_skinny_scaled", x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K,
+                             x.stride(0), out.stride(0), float(alpha), _stream())
+                return None
+            need = int(lib.ra_gemm_wide_scratch(2, M, N, K, 0))
+            scratch = torch.empty(need, dtype=torch.float32, device=x.device) if need else None
+            library.call("ra_gemm_wide_scaled", x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, x.stride(0),
+                         out.stride(0), _ptr(scratch), need, float(alpha), _stream())
+            return None
         if x.dtype != torch.bfloat16:
             raise TypeError("linear_skinny: bfloat16 only")
         if accumulate and out.dtype != torch.float32:

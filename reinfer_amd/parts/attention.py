@@ -74,7 +74,8 @@ class GroupedQueryAttention:
         self.qkv_width = (spec.num_heads + 2 * spec.num_kv_heads) * D
         qn, kn, vn, on = self._names(spec)
         if (key_dim != D or value_dim != D) and (spec.qk_norm or spec.bias):
-            raise ValueError("attention: heads that are laid out with zeros behind them take no head norm and no bias")
+            raise ValueError(f"attention: heads of {key_dim} / {value_dim} are laid out with zeros behind them, which a "
+                             "head norm or a bias does not allow: with those, head sizes go in steps of 16")
 
         def heads_of(w, n, d):           # [n * d, width] -> [n * D, width], zeros behind each head
             if d == D:

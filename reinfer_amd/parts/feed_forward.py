@@ -26,6 +26,7 @@ class SwiGLU:
     adds_in_place = True    # forward(..., resid=) may add the down projection into the stream
     takes_row_scaled = True     # x may be RowScaled: the gate/up product applies the row factor
     emits_for_norm = True       # forward(..., emit=) may fill a NormTarget from the down projection
+    adds_scaled = True          # forward(..., resid=, resid_scale=) adds resid_scale times the result
 
     @staticmethod
     def _names(spec: FeedForwardSpec):
@@ -56,7 +57,8 @@ class SwiGLU:
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = weights[prefix + dn]
 
-    def forward(self, x, batch, resid: Optional[torch.Tensor] = None, emit: Optional[NormTarget] = None):
+    def forward(self, x, batch, resid: Optional[torch.Tensor] = None, emit: Optional[NormTarget] = None,
+                resid_scale: float = 1.0):
         ops = kernels.current()
         x, row_sums = split_input(x)
         T = x.shape[0]
@@ -76,6 +78,9 @@ class SwiGLU:
             ops.silu_mul(gu, act)
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(act, self.w_down):
+            if resid_scale != 1.0:
+                ops.linear_skinny(act, self.w_down, resid, accumulate=True, alpha=resid_scale)
+                return None
             # x += act . Wd^T in the epilogue, which can also prepare the norm that follows
             if emit is not None and emit.finished:
                 done = ops.linear_skinny(act, self.w_down, resid, accumulate=True, finish=emit.finish)

@@ -31,6 +31,7 @@ from .registry import register_mixer
 @register_mixer("matrix_memory")
 class MatrixMemory:
     graph_safe = True       # the scan reads the step's shape from device arrays and leaves state slot -1 alone
+    adds_scaled = True      # forward(..., resid=, resid_scale=) may add the output projection into the stream
 
     NAMES = ("q", "k", "v", "g", "o", "norm", "i", "i.b", "f", "f.b")
 
@@ -68,7 +69,7 @@ class MatrixMemory:
     def cache_need(self) -> StateNeed:
         return StateNeed((self.state_floats,), torch.float32)
 
-    def forward(self, x, batch, cache: LayerCache):
+    def forward(self, x, batch, cache: LayerCache, resid: Optional[torch.Tensor] = None, resid_scale: float = 1.0):
         ops = kernels.current()
         T = x.shape[0]
         H, dk, dv = self.heads, self.key_dim, self.value_dim
@@ -82,6 +83,10 @@ class MatrixMemory:
         act = torch.empty((T, H * dv), dtype=self.dtype, device=x.device)
         ops.head_norm_gate(read, self.norm_weight, True, proj[:, self.offsets[3]:], "sigmoid", self.norm_eps,
                            H, dv, act)
+        can_add = getattr(ops, "can_accumulate", None)
+        if resid is not None and can_add and can_add(act, self.w_o):
+            ops.linear_skinny(act, self.w_o, resid, accumulate=True, alpha=resid_scale)     # x += s * act . Wo^T
+            return None
         out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
         ops.linear(act, self.w_o, out)
         return out

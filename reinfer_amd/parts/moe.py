@@ -37,6 +37,7 @@ from .registry import register_feed_forward
 class MixtureOfExperts:
     graph_safe = True       # routing stays on the device: a decode step with it can be captured
     adds_in_place = True    # forward(..., resid=) may add the down projection into the stream
+    adds_scaled = True      # forward(..., resid=, resid_scale=) adds resid_scale times the result
 
     @classmethod
     def declare_params(cls, spec: FeedForwardSpec, prefix: str) -> List[ParamDecl]:
@@ -90,7 +91,7 @@ class MixtureOfExperts:
         self.w_up = torch.cat([weights[f"{prefix}e{e}.up"] for e in range(self.experts)], dim=0).contiguous()
         self.w_down = torch.cat([weights[f"{prefix}e{e}.down"] for e in range(self.experts)], dim=1).contiguous()
 
-    def _forward_gated(self, x, resid):
+    def _forward_gated(self, x, resid, resid_scale=1.0):
         ops = kernels.current()
         p = self.routing
         T = x.shape[0]
@@ -105,15 +106,20 @@ class MixtureOfExperts:
         ops.moe_silu_gate_scale(gu, act, ids, weights, self.experts, self.ff, self.shared)
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(act, self.w_down):
-            ops.linear_skinny(act, self.w_down, resid, accumulate=True)
+            if resid_scale != 1.0:
+                ops.linear_skinny(act, self.w_down, resid, accumulate=True, alpha=resid_scale)
+            else:
+                ops.linear_skinny(act, self.w_down, resid, accumulate=True)
             return None
         out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
         ops.linear(act, self.w_down, out)
         return out
 
-    def forward(self, x, batch, resid: Optional[torch.Tensor] = None):
+    def forward(self, x, batch, resid: Optional[torch.Tensor] = None, resid_scale: float = 1.0):
         if self.gated:
-            return self._forward_gated(x, resid)
+            return self._forward_gated(x, resid, resid_scale)
+        if resid_scale != 1.0:
+            resid = None                    # the ungated form adds its result as it is: the caller scales it
         ops = kernels.current()
         T = x.shape[0]
         n = self.experts * self.ff

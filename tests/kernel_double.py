@@ -357,8 +357,8 @@ class KernelDouble:
         ss, eps, width = row_sums
         return torch.rsqrt(ss.double().sum(0) / width + eps).float()
 
-    def linear_skinny(self, x, weight, out, bias=None, accumulate=False, row_sums=None, emit=None):
-        y = x.float() @ weight.float().T
+    def linear_skinny(self, x, weight, out, bias=None, accumulate=False, row_sums=None, emit=None, alpha=1.0):
+        y = (x.float() @ weight.float().T) * alpha
         if row_sums is not None:
             y = y * self._rstd(row_sums)[:, None]
         if bias is not None:

@@ -213,3 +213,20 @@ def test_scaled_adds_and_embedding(dtype):
     ref.embed(table, ids, a, scale=16.0)
     ops.embed(table.to(DEV), ids.to(DEV), b, scale=16.0)
     close(b, a, 1e-7, "embed")
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64, 65, 100, 128, 200, 2048])
+@pytest.mark.parametrize("N,K", [(256, 128), (2048, 2048), (4096, 1024), (96, 144)])
+def test_accumulating_product_with_a_factor(M, N, K):
+    """out += alpha * (x . W^T) through whichever product takes the row count: both weight-streaming kernels, the
+    one that cuts K into ranges, and the library's."""
+    ops = kernels.current()
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(DEV)
+    out = torch.randn(M, N, generator=g).to(DEV)
+    if not ops.can_accumulate(x, w):
+        pytest.skip("no accumulating product at this row count")
+    ref = out.double() + 0.3 * (x.double() @ w.double().T)
+    ops.linear_skinny(x, w, out, accumulate=True, alpha=0.3)
+    close(out, ref, 2e-5, "scaled accumulate")
