@@ -43,89 +43,194 @@ __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log
 __device__ __forceinline__ float logsigmoid_f(float x) { return -softplus_f(-x); }
 
 // ---------------------------------------------------------------------------
-// Matrix memory. lg[t, h] = log input gate a, lg[t, H + h] = log forget gate b (prepared below).
+// The scan of either mixer. A workgroup (up to 4 waves: 32 or 8 columns of one head of one request) walks the
+// request's tokens in chunks: the chunk's k and q rows of the head (as floats, q scaled), the v entries of the
+// workgroup's columns and the two gate values a token are fetched into registers while the chunk before is
+// computed, written to LDS behind it, and read from there token by token (a lane's NPL elements of k and of q
+// are one run of LDS, rows padded so that the 16-byte reads of a wave fall on different banks). One barrier a
+// chunk; every wave of the workgroup takes part in the staging, also those past the head's last column.
+//
+// Matrix memory (MEMORY): gt[t, h] = log input gate a, gt[t, H + h] = log forget gate b (prepared below).
 //   m' = max(b + m, a);  keep = exp(b + m - m');  take = exp(a - m')
 //   S <- keep S + take k v^T;  n <- keep n + take k;  o = S^T q / (max(|n . q|, exp(-m')) + eps)
+// Gated delta rule: gt[t, h] = beta, gt[t, H + h] = decay g (prepared below).
+//   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// computed from the state before the decay: a = S^T k, b = S^T q, kq = k . q in one butterfly, then
+// u = beta (v - g a), o = g b + u kq, S <- g S + k u.
 // ---------------------------------------------------------------------------
-template <typename TA, int R, int NPL>
-__global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
-    const TA* __restrict__ proj, int ld, int q_off, int k_off, int v_off, const float* __restrict__ lg,
-    float* __restrict__ state, long slot_stride, const int* __restrict__ cu_tokens,
-    const int* __restrict__ state_slots, const int* __restrict__ fresh, int H, int dk, int dv, int waves_per_head,
-    int wave_floats, float q_scale, float denom_eps, float* __restrict__ out) {
+#define SCAN_KQ_REGS 8         // k (and q) values a thread fetches for a chunk
+#define SCAN_V_REGS 2
+#define SCAN_CHUNK_MAX 16
+#define SCAN_LDS_FLOATS 6144   // of one of the two buffers
+
+struct ScanArgs {
+  const void* q; const void* k; const void* v;     // column 0 of each in row 0; rows ld elements apart
+  int ld;
+  int q_heads;                                       // heads of q and k (value heads share them in equal runs)
+  const float* gates;                                // [T, 2 H]
+  float* state; long slot_stride;
+  const int* cu_tokens; const int* state_slots; const int* fresh;
+  int H, dk, dv, waves_per_head, wave_floats, chunk;
+  float q_scale, denom_eps;
+  float* out;
+};
+
+template <typename TA, int R, int NPL, bool MEMORY>
+__global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
   constexpr int CPW = RA_WAVE / R;
+  constexpr int PITCH = NPL + 4;                     // floats of a lane's run of k (or q) in LDS, padded
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int seq = blockIdx.x, head = blockIdx.y;
-  const int lane = threadIdx.x & (RA_WAVE - 1);
-  const int w = blockIdx.z * (blockDim.x / RA_WAVE) + threadIdx.x / RA_WAVE;
-  if (w >= waves_per_head) return;           // whole waves leave; there is no barrier below
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int lane = tid & (RA_WAVE - 1);
+  const int waves = nthreads / RA_WAVE;
+  const int cols = waves * CPW;                      // columns of this workgroup
+  const int w = blockIdx.z * waves + tid / RA_WAVE;
+  const bool active = w < p.waves_per_head;
   const int c = lane / R, r = lane % R;
   const int col = w * CPW + c;
-  const bool col_ok = col < dv;
-  const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
-  const int slot = state_slots[seq];
-  const int ow = H * dv;
-  if (slot < 0) {                            // a padding row: no state, a defined result
+  const bool col_ok = active && col < p.dv;
+  const int first = p.cu_tokens[seq], last = p.cu_tokens[seq + 1];
+  const int slot = p.state_slots[seq];
+  const int ow = p.H * p.dv;
+  const int H = p.H, dk = p.dk, dv = p.dv, CT = p.chunk;
+  if (slot < 0) {                                    // a padding row: no state, a defined result
     if (col_ok && r == 0)
-      for (int t = first; t < last; ++t) out[(size_t)t * ow + head * dv + col] = 0.f;
+      for (int t = first; t < last; ++t) p.out[(size_t)t * ow + head * dv + col] = 0.f;
     return;
   }
   if (first >= last) return;
-  float* st = state + (size_t)slot * slot_stride + (size_t)(head * waves_per_head + w) * wave_floats;
-  const bool zero = fresh[seq] != 0;
-  float S[NPL], n[NPL];
+  // LDS: two buffers of [CT][2][R][PITCH] k and q, [CT][cols] v, [CT][2] gates
+  const int kq_floats = CT * 2 * R * PITCH, v_floats = CT * cols;
+  const int buf_floats = kq_floats + v_floats + CT * 2;
+  for (int i = tid; i < 2 * buf_floats; i += nthreads) lds[i] = 0.f;      // the padding stays zero
+  const int qh = head / (H / p.q_heads);
+  const TA* qg = (const TA*)p.q + (size_t)qh * dk;
+  const TA* kg = (const TA*)p.k + (size_t)qh * dk;
+  const TA* vg = (const TA*)p.v + (size_t)head * dv + (size_t)blockIdx.z * cols;
+  const int v_left = dv - blockIdx.z * cols;         // columns of this workgroup that exist
+  float fk[SCAN_KQ_REGS], fq[SCAN_KQ_REGS], fv[SCAN_V_REGS], fg = 0.f;
+  auto fetch = [&](int t0) {                         // chunk starting at token t0 -> registers
+    const int n = min(CT, last - t0);
+#pragma unroll
+    for (int j = 0; j < SCAN_KQ_REGS; ++j) {
+      const int idx = tid + j * nthreads;
+      const int t = idx / dk, e = idx - t * dk;
+      fk[j] = fq[j] = 0.f;
+      if (t < n) {
+        const size_t row = (size_t)(t0 + t) * p.ld;
+        fk[j] = to_f32(kg[row + e]);
+        fq[j] = to_f32(qg[row + e]) * p.q_scale;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < SCAN_V_REGS; ++j) {
+      const int idx = tid + j * nthreads;
+      const int t = idx / cols, cc = idx - t * cols;
+      fv[j] = (t < n && cc < v_left) ? to_f32(vg[(size_t)(t0 + t) * p.ld + cc]) : 0.f;
+    }
+    if (tid < 2 * CT) {
+      const int t = tid >> 1;
+      fg = t < n ? p.gates[(size_t)(t0 + t) * 2 * H + (tid & 1) * H + head] : 0.f;
+    }
+  };
+  auto stage = [&](float* buf) {                     // registers -> LDS
+#pragma unroll
+    for (int j = 0; j < SCAN_KQ_REGS; ++j) {
+      const int idx = tid + j * nthreads;
+      const int t = idx / dk, e = idx - t * dk;
+      if (t < CT) {
+        float* row = buf + (size_t)t * 2 * R * PITCH + (e / NPL) * PITCH + (e % NPL);
+        row[0] = fk[j];
+        row[R * PITCH] = fq[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < SCAN_V_REGS; ++j) {
+      const int idx = tid + j * nthreads;
+      if (idx < v_floats) buf[kq_floats + idx] = fv[j];
+    }
+    if (tid < 2 * CT) buf[kq_floats + v_floats + tid] = fg;
+  };
+  float* st = p.state + (size_t)slot * p.slot_stride + (size_t)(head * p.waves_per_head + (active ? w : 0)) * p.wave_floats;
+  const bool zero = p.fresh[seq] != 0;
+  float S[NPL], nrm[NPL];
+  float m = 0.f;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
-    S[i] = zero ? 0.f : st[i * RA_WAVE + lane];
-    n[i] = zero ? 0.f : st[NPL * RA_WAVE + i * R + r];
+    S[i] = (zero || !active) ? 0.f : st[i * RA_WAVE + lane];
+    nrm[i] = 0.f;
+    if (MEMORY && !zero && active) nrm[i] = st[NPL * RA_WAVE + i * R + r];
   }
-  float m = zero ? 0.f : st[NPL * RA_WAVE + NPL * R];
-  const TA* qp = proj + q_off + head * dk;
-  const TA* kp = proj + k_off + head * dk;
-  const TA* vp = proj + v_off + head * dv + (col_ok ? col : 0);
-  float nk[NPL], nq[NPL], nv, na, nb;
-  auto fetch = [&](int t) {
-    const size_t row = (size_t)t * ld;
-#pragma unroll
-    for (int i = 0; i < NPL; ++i) {
-      const int e = i * R + r;
-      nk[i] = e < dk ? to_f32(kp[row + e]) : 0.f;
-      nq[i] = e < dk ? to_f32(qp[row + e]) : 0.f;
-    }
-    nv = col_ok ? to_f32(vp[row]) : 0.f;
-    na = lg[(size_t)t * 2 * H + head];
-    nb = lg[(size_t)t * 2 * H + H + head];
-  };
+  if (MEMORY && !zero && active) m = st[NPL * RA_WAVE + NPL * R];
   fetch(first);
-  for (int t = first; t < last; ++t) {
-    float k[NPL], q[NPL];
+  __syncthreads();                                   // the zero fill is done
+  stage(lds);
+  __syncthreads();
+  int which = 0;
+  for (int t0 = first; t0 < last; t0 += CT) {
+    const bool more = t0 + CT < last;
+    if (more) fetch(t0 + CT);
+    const float* buf = lds + (size_t)which * buf_floats;
+    const int n = min(CT, last - t0);
+    if (active) {
+#pragma unroll 2
+      for (int tt = 0; tt < n; ++tt) {
+        const float* kp = buf + (size_t)tt * 2 * R * PITCH + r * PITCH;
+        const float* qp = kp + R * PITCH;
+        float k[NPL], q[NPL];
 #pragma unroll
-    for (int i = 0; i < NPL; ++i) { k[i] = nk[i]; q[i] = nq[i] * q_scale; }
-    const float v = nv, a = na, b = nb;
-    if (t + 1 < last) fetch(t + 1);
-    const float m_new = fmaxf(b + m, a);
-    const float keep = expf(b + m - m_new);
-    const float take = expf(a - m_new);
-    m = m_new;
-    float ps = 0.f, pn = 0.f;
+        for (int i = 0; i < NPL; ++i) { k[i] = kp[i]; q[i] = qp[i]; }
+        const float v = buf[kq_floats + tt * cols + (tid / RA_WAVE) * CPW + c];
+        const float g0 = buf[kq_floats + v_floats + 2 * tt], g1 = buf[kq_floats + v_floats + 2 * tt + 1];
+        float o;
+        if (MEMORY) {
+          const float m_new = fmaxf(g1 + m, g0);
+          const float keep = expf(g1 + m - m_new);
+          const float take = expf(g0 - m_new);
+          m = m_new;
+          float ps = 0.f, pn = 0.f;
 #pragma unroll
-    for (int i = 0; i < NPL; ++i) {
-      const float tk = take * k[i];
-      n[i] = keep * n[i] + tk;
-      S[i] = keep * S[i] + tk * v;
-      ps += S[i] * q[i];
-      pn += n[i] * q[i];
+          for (int i = 0; i < NPL; ++i) {
+            const float tk = take * k[i];
+            nrm[i] = keep * nrm[i] + tk;
+            S[i] = keep * S[i] + tk * v;
+            ps += S[i] * q[i];
+            pn += nrm[i] * q[i];
+          }
+          ps = group_sum<R>(ps);
+          pn = group_sum<R>(pn);
+          o = ps / (fmaxf(fabsf(pn), expf(-m)) + p.denom_eps);
+        } else {
+          float pa = 0.f, pb = 0.f, pkq = 0.f;
+#pragma unroll
+          for (int i = 0; i < NPL; ++i) {
+            pa += S[i] * k[i];
+            pb += S[i] * q[i];
+            pkq += k[i] * q[i];
+          }
+          pa = group_sum<R>(pa);
+          pb = group_sum<R>(pb);
+          pkq = group_sum<R>(pkq);
+          const float u = g0 * (v - g1 * pa);
+#pragma unroll
+          for (int i = 0; i < NPL; ++i) S[i] = g1 * S[i] + k[i] * u;
+          o = g1 * pb + u * pkq;
+        }
+        if (col_ok && r == 0) p.out[(size_t)(t0 + tt) * ow + head * dv + col] = o;
+      }
     }
-    ps = group_sum<R>(ps);
-    pn = group_sum<R>(pn);
-    const float den = fmaxf(fabsf(pn), expf(-m)) + denom_eps;
-    if (col_ok && r == 0) out[(size_t)t * ow + head * dv + col] = ps / den;
+    if (more) stage(lds + (size_t)(which ^ 1) * buf_floats);
+    __syncthreads();
+    which ^= 1;
   }
+  if (!active) return;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     st[i * RA_WAVE + lane] = S[i];
-    if (c == 0) st[NPL * RA_WAVE + i * R + r] = n[i];
+    if (MEMORY && c == 0) st[NPL * RA_WAVE + i * R + r] = nrm[i];
   }
-  if (lane == 0) st[NPL * RA_WAVE + NPL * R] = m;
+  if (MEMORY && lane == 0) st[NPL * RA_WAVE + NPL * R] = m;
 }
 
 // lg[t, h] <- cap tanh((z + bias) / cap);  lg[t, H + h] <- log sigmoid(cap tanh((z + bias) / cap)), in place
@@ -137,82 +242,6 @@ __global__ void matrix_memory_gates_kernel(float* __restrict__ lg, const float* 
   float z = lg[i] + bias[j];
   if (cap > 0.f) z = cap * tanhf(z / cap);
   lg[i] = j < H ? z : logsigmoid_f(z);
-}
-
-// ---------------------------------------------------------------------------
-// Gated delta rule. gb[t, h] = beta, gb[t, H + h] = decay g (prepared below); qkv float [T, q | k | v].
-//   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
-// computed from the state before the decay: a = S^T k, b = S^T q, kq = k . q in one butterfly, then
-// u = beta (v - g a), o = g b + u kq, S <- g S + k u.
-// ---------------------------------------------------------------------------
-template <int R, int NPL>
-__global__ __launch_bounds__(256) void delta_rule_scan_kernel(
-    const float* __restrict__ qkv, int ld, const float* __restrict__ gb, float* __restrict__ state, long slot_stride,
-    const int* __restrict__ cu_tokens, const int* __restrict__ state_slots, const int* __restrict__ fresh, int H,
-    int G, int dk, int dv, int waves_per_head, float* __restrict__ out) {
-  constexpr int CPW = RA_WAVE / R;
-  const int seq = blockIdx.x, head = blockIdx.y;
-  const int lane = threadIdx.x & (RA_WAVE - 1);
-  const int w = blockIdx.z * (blockDim.x / RA_WAVE) + threadIdx.x / RA_WAVE;
-  if (w >= waves_per_head) return;
-  const int c = lane / R, r = lane % R;
-  const int col = w * CPW + c;
-  const bool col_ok = col < dv;
-  const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
-  const int slot = state_slots[seq];
-  const int ow = H * dv;
-  if (slot < 0) {
-    if (col_ok && r == 0)
-      for (int t = first; t < last; ++t) out[(size_t)t * ow + head * dv + col] = 0.f;
-    return;
-  }
-  if (first >= last) return;
-  float* st = state + (size_t)slot * slot_stride + (size_t)(head * waves_per_head + w) * (NPL * RA_WAVE);
-  const bool zero = fresh[seq] != 0;
-  float S[NPL];
-#pragma unroll
-  for (int i = 0; i < NPL; ++i) S[i] = zero ? 0.f : st[i * RA_WAVE + lane];
-  const int kh = head / (H / G);
-  const float* qp = qkv + kh * dk;
-  const float* kp = qkv + G * dk + kh * dk;
-  const float* vp = qkv + 2 * G * dk + head * dv + (col_ok ? col : 0);
-  float nk[NPL], nq[NPL], nv, nbeta, ng;
-  auto fetch = [&](int t) {
-    const size_t row = (size_t)t * ld;
-#pragma unroll
-    for (int i = 0; i < NPL; ++i) {
-      const int e = i * R + r;
-      nk[i] = e < dk ? kp[row + e] : 0.f;
-      nq[i] = e < dk ? qp[row + e] : 0.f;
-    }
-    nv = col_ok ? vp[row] : 0.f;
-    nbeta = gb[(size_t)t * 2 * H + head];
-    ng = gb[(size_t)t * 2 * H + H + head];
-  };
-  fetch(first);
-  for (int t = first; t < last; ++t) {
-    float k[NPL], q[NPL];
-#pragma unroll
-    for (int i = 0; i < NPL; ++i) { k[i] = nk[i]; q[i] = nq[i]; }
-    const float v = nv, beta = nbeta, g = ng;
-    if (t + 1 < last) fetch(t + 1);
-    float pa = 0.f, pb = 0.f, pkq = 0.f;
-#pragma unroll
-    for (int i = 0; i < NPL; ++i) {
-      pa += S[i] * k[i];
-      pb += S[i] * q[i];
-      pkq += k[i] * q[i];
-    }
-    pa = group_sum<R>(pa);
-    pb = group_sum<R>(pb);
-    pkq = group_sum<R>(pkq);
-    const float u = beta * (v - g * pa);
-#pragma unroll
-    for (int i = 0; i < NPL; ++i) S[i] = g * S[i] + k[i] * u;
-    if (col_ok && r == 0) out[(size_t)t * ow + head * dv + col] = g * pb + u * pkq;
-  }
-#pragma unroll
-  for (int i = 0; i < NPL; ++i) st[i * RA_WAVE + lane] = S[i];
 }
 
 // gb[t, h] <- sigmoid(b);  gb[t, H + h] <- exp(-exp(A_log[h]) softplus(a + dt_bias[h])), in place
@@ -355,27 +384,39 @@ struct MeanInputs {
   const void* x[MEAN_MAX];
   const float* w[MEAN_MAX];
 };
-template <typename TA>
-__global__ void normed_mean_kernel(MeanInputs in, int n, float eps, int h, TA* __restrict__ out,
-                                   float* __restrict__ resid, float scale) {
-  __shared__ float red[17];
+template <typename TA, int N>
+__global__ void normed_mean_kernel(MeanInputs in, float eps, int h, TA* __restrict__ out, float* __restrict__ resid,
+                                   float scale) {
+  __shared__ float red[N][17];
   const size_t row = (size_t)blockIdx.x * h;
-  float rstd[MEAN_MAX];
-  for (int i = 0; i < n; ++i) {
-    const TA* x = (const TA*)in.x[i] + row;
-    float ss = 0.f;
-    for (int e = threadIdx.x; e < h; e += blockDim.x) {
-      const float v = to_f32(x[e]);
-      ss += v * v;
+  const int lane = threadIdx.x & (RA_WAVE - 1), wave = threadIdx.x / RA_WAVE, nwave = blockDim.x / RA_WAVE;
+  float ss[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) ss[i] = 0.f;
+  for (int e = threadIdx.x; e < h; e += blockDim.x) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const float v = to_f32(((const TA*)in.x[i])[row + e]);
+      ss[i] += v * v;
     }
-    ss = block_sum(ss, red);
-    rstd[i] = 1.f / sqrtf(ss / (float)h + eps);
   }
-  const float inv = 1.f / (float)n;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    ss[i] = wave_sum(ss[i]);
+    if (lane == 0) red[i][wave] = ss[i];
+  }
+  __syncthreads();
+  float rstd[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    float t = 0.f;
+    for (int w = 0; w < nwave; ++w) t += red[i][w];          // fixed order
+    rstd[i] = 1.f / sqrtf(t / (float)h + eps) * (1.f / (float)N);
+  }
   for (int e = threadIdx.x; e < h; e += blockDim.x) {
     float y = 0.f;
-    for (int i = 0; i < n; ++i) y += to_f32(((const TA*)in.x[i])[row + e]) * rstd[i] * in.w[i][e];
-    y *= inv;
+#pragma unroll
+    for (int i = 0; i < N; ++i) y += to_f32(((const TA*)in.x[i])[row + e]) * rstd[i] * in.w[i][e];
     if (resid) resid[row + e] += scale * y;
     else out[row + e] = from_f32<TA>(y);
   }
@@ -395,14 +436,41 @@ extern "C" long ra_scan_state_floats(int kind, int heads, int key_dim, int value
 namespace {
 struct ScanLaunch {
   dim3 grid;
-  int threads;
+  int threads, chunk;
+  size_t lds;
 };
-ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads) {
+ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int dk) {
   const int wpb = g.waves < 4 ? g.waves : 4;           // waves a workgroup
   ScanLaunch L;
   L.threads = wpb * RA_WAVE;
   L.grid = dim3(n_seqs, heads, (g.waves + wpb - 1) / wpb);
+  const int cols = wpb * g.CPW;
+  const int per_token = 2 * g.R * (g.NPL + 4) + cols + 2;
+  int ct = SCAN_CHUNK_MAX;
+  if (ct > SCAN_KQ_REGS * L.threads / dk) ct = SCAN_KQ_REGS * L.threads / dk;
+  if (ct > SCAN_V_REGS * L.threads / cols) ct = SCAN_V_REGS * L.threads / cols;
+  if (ct > SCAN_LDS_FLOATS / per_token) ct = SCAN_LDS_FLOATS / per_token;
+  if (ct > L.threads / 2) ct = L.threads / 2;
+  if (ct < 1) ct = 1;
+  L.chunk = ct;
+  L.lds = (size_t)2 * ((size_t)ct * per_token) * sizeof(float);
   return L;
+}
+
+template <typename TA, bool MEMORY>
+int scan_dispatch(const ScanGeom& g, const ScanLaunch& L, const ScanArgs& a, hipStream_t stream) {
+#define RA_SCAN(R, NPL) scan_kernel<TA, R, NPL, MEMORY><<<L.grid, L.threads, L.lds, stream>>>(a)
+#define RA_SCAN_N(R)                               \
+  do {                                             \
+    if (g.NPL == 2) RA_SCAN(R, 2);                 \
+    else if (g.NPL == 4) RA_SCAN(R, 4);            \
+    else if (g.NPL == 8) RA_SCAN(R, 8);            \
+    else RA_SCAN(R, 16);                           \
+  } while (0)
+  if (g.R == 8) RA_SCAN_N(8); else RA_SCAN_N(32);
+#undef RA_SCAN_N
+#undef RA_SCAN
+  return 0;
 }
 }  // namespace
 
@@ -419,30 +487,22 @@ extern "C" int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, in
   RA_CHECK(slot_stride >= (long)heads * g.waves * g.wave_floats, "matrix_memory_scan: a state slot of %ld floats, need %ld",
            slot_stride, (long)heads * g.waves * g.wave_floats);
   RA_CHECK(heads <= 65535, "matrix_memory_scan: %d heads in one launch", heads);
+  RA_CHECK(act_dtype == RA_F32 || act_dtype == RA_BF16, "matrix_memory_scan: unknown dtype tag %d", act_dtype);
   const long n = (long)n_tokens * 2 * heads;
   matrix_memory_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(gates, gate_bias, heads, gate_cap, n);
   RA_LAUNCH_CHECK("matrix_memory_gates");
-  const ScanLaunch L = scan_launch(g, n_seqs, heads);
-#define RA_MM(TA, R, NPL)                                                                                         \
-  matrix_memory_scan_kernel<TA, R, NPL><<<L.grid, L.threads, 0, stream>>>(                                        \
-      (const TA*)proj, ld, q_off, k_off, v_off, gates, state, slot_stride, cu_tokens, state_slots, fresh, heads,  \
-      key_dim, value_dim, g.waves, g.wave_floats, q_scale, denom_eps, out)
-#define RA_MM_N(TA, R)                                  \
-  do {                                                  \
-    if (g.NPL == 2) RA_MM(TA, R, 2);                    \
-    else if (g.NPL == 4) RA_MM(TA, R, 4);               \
-    else if (g.NPL == 8) RA_MM(TA, R, 8);               \
-    else RA_MM(TA, R, 16);                              \
-  } while (0)
-  if (act_dtype == RA_F32) {
-    if (g.R == 8) RA_MM_N(float, 8); else RA_MM_N(float, 32);
-  } else if (act_dtype == RA_BF16) {
-    if (g.R == 8) RA_MM_N(bf16_t, 8); else RA_MM_N(bf16_t, 32);
-  } else {
-    return ra_fail("matrix_memory_scan: unknown dtype tag %d", act_dtype);
-  }
-#undef RA_MM_N
-#undef RA_MM
+  const ScanLaunch L = scan_launch(g, n_seqs, heads, key_dim);
+  const size_t es = act_dtype == RA_F32 ? 4 : 2;
+  ScanArgs a = {};
+  a.q = (const char*)proj + (size_t)q_off * es;
+  a.k = (const char*)proj + (size_t)k_off * es;
+  a.v = (const char*)proj + (size_t)v_off * es;
+  a.ld = ld; a.q_heads = heads; a.gates = gates; a.state = state; a.slot_stride = slot_stride;
+  a.cu_tokens = cu_tokens; a.state_slots = state_slots; a.fresh = fresh;
+  a.H = heads; a.dk = key_dim; a.dv = value_dim; a.waves_per_head = g.waves; a.wave_floats = g.wave_floats;
+  a.chunk = L.chunk; a.q_scale = q_scale; a.denom_eps = denom_eps; a.out = out;
+  if (act_dtype == RA_F32) scan_dispatch<float, true>(g, L, a, stream);
+  else scan_dispatch<bf16_t, true>(g, L, a, stream);
   RA_LAUNCH_CHECK("matrix_memory_scan");
   return 0;
 }
@@ -494,21 +554,16 @@ extern "C" int ra_delta_rule_scan(const float* qkv, int ld, float* gates, const 
   const long n = (long)n_tokens * 2 * heads;
   delta_rule_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(gates, a_log, dt_bias, heads, n);
   RA_LAUNCH_CHECK("delta_rule_gates");
-  const ScanLaunch L = scan_launch(g, n_seqs, heads);
-#define RA_DS(R, NPL)                                                                                          \
-  delta_rule_scan_kernel<R, NPL><<<L.grid, L.threads, 0, stream>>>(qkv, ld, gates, state, slot_stride, cu_tokens, \
-                                                                  state_slots, fresh, heads, key_heads, key_dim,   \
-                                                                  value_dim, g.waves, out)
-#define RA_DS_N(R)                               \
-  do {                                           \
-    if (g.NPL == 2) RA_DS(R, 2);                 \
-    else if (g.NPL == 4) RA_DS(R, 4);            \
-    else if (g.NPL == 8) RA_DS(R, 8);            \
-    else RA_DS(R, 16);                           \
-  } while (0)
-  if (g.R == 8) RA_DS_N(8); else RA_DS_N(32);
-#undef RA_DS_N
-#undef RA_DS
+  const ScanLaunch L = scan_launch(g, n_seqs, heads, key_dim);
+  ScanArgs a = {};
+  a.q = qkv;
+  a.k = qkv + (size_t)key_heads * key_dim;
+  a.v = qkv + (size_t)2 * key_heads * key_dim;
+  a.ld = ld; a.q_heads = key_heads; a.gates = gates; a.state = state; a.slot_stride = slot_stride;
+  a.cu_tokens = cu_tokens; a.state_slots = state_slots; a.fresh = fresh;
+  a.H = heads; a.dk = key_dim; a.dv = value_dim; a.waves_per_head = g.waves; a.wave_floats = g.wave_floats;
+  a.chunk = L.chunk; a.q_scale = 1.f; a.denom_eps = 0.f; a.out = out;
+  scan_dispatch<float, false>(g, L, a, stream);
   RA_LAUNCH_CHECK("delta_rule_scan");
   return 0;
 }
@@ -543,12 +598,20 @@ extern "C" int ra_normed_mean(const void* const* xs, const float* const* ws, int
     in.x[i] = i < n ? xs[i] : nullptr;
     in.w[i] = i < n ? ws[i] : nullptr;
   }
-  if (act_dtype == RA_F32)
-    normed_mean_kernel<float><<<n_tokens, 256, 0, stream>>>(in, n, eps, hidden, (float*)out, resid, scale);
-  else if (act_dtype == RA_BF16)
-    normed_mean_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(in, n, eps, hidden, (bf16_t*)out, resid, scale);
-  else
-    return ra_fail("normed_mean: unknown dtype tag %d", act_dtype);
+  const int threads = hidden >= 2048 ? 512 : 256;
+#define RA_NM(TA, N) normed_mean_kernel<TA, N><<<n_tokens, threads, 0, stream>>>(in, eps, hidden, (TA*)out, resid, scale)
+#define RA_NM_N(TA)                 \
+  do {                              \
+    if (n == 1) RA_NM(TA, 1);       \
+    else if (n == 2) RA_NM(TA, 2);  \
+    else if (n == 3) RA_NM(TA, 3);  \
+    else RA_NM(TA, 4);              \
+  } while (0)
+  if (act_dtype == RA_F32) RA_NM_N(float);
+  else if (act_dtype == RA_BF16) RA_NM_N(bf16_t);
+  else return ra_fail("normed_mean: unknown dtype tag %d", act_dtype);
+#undef RA_NM_N
+#undef RA_NM
   RA_LAUNCH_CHECK("normed_mean");
   return 0;
 }
