@@ -5,8 +5,7 @@
 //
 // The scans. A column of the state (one value index) evolves on its own given the token's k, q and gates, so
 // the columns are spread over lanes, waves and workgroups and every wave walks the request's tokens in order:
-// R lanes share a column, lane r of them holding elements r, r + R, ... of it (NPL a lane); a wave holds
-// 64 / R columns. The two dot products a token needs (with k or n, and with q) are sums over a lane's elements
+// R lanes share a column, each holding a run of NPL of its elements; a wave holds 64 / R columns. The two dot products a token needs (with k or n, and with q) are sums over a lane's elements
 // and a butterfly over the R lanes. The next token's operands are asked for before the current token's
 // arithmetic. The state of a request lives in its slot in the waves' own order, [NPL][64] floats a wave, so
 // that loading and storing it are whole lines; nothing else reads it.
@@ -23,19 +22,32 @@ struct ScanGeom {
 // kind 0: matrix memory (S, the normaliser n once a wave, the running maximum m); kind 1: delta rule (S)
 bool scan_geom(int kind, int dk, int dv, ScanGeom* g) {
   if (dk <= 0 || dv <= 0 || dk > 512) return false;
-  g->R = dk <= 128 ? 8 : 32;
+  // at most 8 elements a lane: the per-token chain of multiply-adds stays short, and a head has enough waves to
+  // spread over the chip when one request's prompt is all there is
+  g->R = dk <= 32 ? 8 : dk <= 128 ? 16 : dk <= 256 ? 32 : 64;
   const int per = (dk + g->R - 1) / g->R;
-  g->NPL = per <= 2 ? 2 : per <= 4 ? 4 : per <= 8 ? 8 : 16;
+  g->NPL = per <= 2 ? 2 : per <= 4 ? 4 : 8;
   g->CPW = RA_WAVE / g->R;
   g->waves = (dv + g->CPW - 1) / g->CPW;
   g->wave_floats = g->NPL * RA_WAVE + (kind == 0 ? g->NPL * g->R + 4 : 0);
   return true;
 }
 
+// Sum over runs of R neighbouring lanes, every lane of a run getting the sum. Inside a row of 16 lanes the
+// exchanges are DPP operands of the adds (pairs, quads, the mirrored half row and row); only beyond 16 lanes does
+// a value travel through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
 template <int R>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int m = R / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, RA_WAVE);
+  v += dpp_move<0xB1>(v);                    // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);                    // quad_perm [2, 3, 0, 1]
+  v += dpp_move<0x141>(v);                   // row_half_mirror: the other quad of the 8
+  if (R >= 16) v += dpp_move<0x140>(v);      // row_mirror: the other half of the 16
+  if (R >= 32) v += __shfl_xor(v, 16, RA_WAVE);
+  if (R >= 64) v += __shfl_xor(v, 32, RA_WAVE);
   return v;
 }
 
@@ -50,8 +62,8 @@ __device__ __forceinline__ float logsigmoid_f(float x) { return -softplus_f(-x);
 // are one run of LDS, rows padded so that the 16-byte reads of a wave fall on different banks). One barrier a
 // chunk; every wave of the workgroup takes part in the staging, also those past the head's last column.
 //
-// Matrix memory (MEMORY): gt[t, h] = log input gate a, gt[t, H + h] = log forget gate b (prepared below).
-//   m' = max(b + m, a);  keep = exp(b + m - m');  take = exp(a - m')
+// Matrix memory (MEMORY): gt[t, j H + h], j = 0, 1, 2: keep = exp(b + m - m'), take = exp(a - m') and exp(-m') with
+// m' = max(b + m, a) the running maximum of the log gates (all three prepared below, where the maximum is kept)
 //   S <- keep S + take k v^T;  n <- keep n + take k;  o = S^T q / (max(|n . q|, exp(-m')) + eps)
 // Gated delta rule: gt[t, h] = beta, gt[t, H + h] = decay g (prepared below).
 //   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
@@ -67,7 +79,7 @@ struct ScanArgs {
   const void* q; const void* k; const void* v;     // column 0 of each in row 0; rows ld elements apart
   int ld;
   int q_heads;                                       // heads of q and k (value heads share them in equal runs)
-  const float* gates;                                // [T, 2 H]
+  const float* gates;                                // [T, NG H], NG = 3 (matrix memory) or 2 (delta rule)
   float* state; long slot_stride;
   const int* cu_tokens; const int* state_slots; const int* fresh;
   int H, dk, dv, waves_per_head, wave_floats, chunk;
@@ -79,6 +91,7 @@ template <typename TA, int R, int NPL, bool MEMORY>
 __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
   constexpr int CPW = RA_WAVE / R;
   constexpr int PITCH = NPL + 4;                     // floats of a lane's run of k (or q) in LDS, padded
+  constexpr int NG = MEMORY ? 3 : 2;                 // gate values a token
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int seq = blockIdx.x, head = blockIdx.y;
   const int tid = threadIdx.x, nthreads = blockDim.x;
@@ -100,9 +113,9 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     return;
   }
   if (first >= last) return;
-  // LDS: two buffers of [CT][2][R][PITCH] k and q, [CT][cols] v, [CT][2] gates
+  // LDS: two buffers of [CT][2][R][PITCH] k and q, [CT][cols] v, [CT][NG] gates
   const int kq_floats = CT * 2 * R * PITCH, v_floats = CT * cols;
-  const int buf_floats = kq_floats + v_floats + CT * 2;
+  const int buf_floats = kq_floats + v_floats + CT * NG;
   for (int i = tid; i < 2 * buf_floats; i += nthreads) lds[i] = 0.f;      // the padding stays zero
   const int qh = head / (H / p.q_heads);
   const TA* qg = (const TA*)p.q + (size_t)qh * dk;
@@ -110,39 +123,48 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
   const TA* vg = (const TA*)p.v + (size_t)head * dv + (size_t)blockIdx.z * cols;
   const int v_left = dv - blockIdx.z * cols;         // columns of this workgroup that exist
   float fk[SCAN_KQ_REGS], fq[SCAN_KQ_REGS], fv[SCAN_V_REGS], fg = 0.f;
+  // what this thread fetches for a chunk is the same for every chunk: token (of the chunk), offset behind the
+  // chunk's first row, and place in LDS are worked out once
+  int kq_t[SCAN_KQ_REGS], kq_g[SCAN_KQ_REGS], kq_l[SCAN_KQ_REGS];
+#pragma unroll
+  for (int j = 0; j < SCAN_KQ_REGS; ++j) {
+    const int idx = tid + j * nthreads;
+    const int t = idx / dk, e = idx - t * dk;
+    kq_t[j] = t < CT ? t : SCAN_CHUNK_MAX;           // past the chunk: never fetched, never stored
+    kq_g[j] = t * p.ld + e;
+    kq_l[j] = t * 2 * R * PITCH + (e / NPL) * PITCH + (e % NPL);
+  }
+  int v_t[SCAN_V_REGS], v_g[SCAN_V_REGS];
+#pragma unroll
+  for (int j = 0; j < SCAN_V_REGS; ++j) {
+    const int idx = tid + j * nthreads;
+    const int t = idx / cols, cc = idx - t * cols;
+    v_t[j] = (t < CT && cc < v_left) ? t : SCAN_CHUNK_MAX;
+    v_g[j] = t * p.ld + cc;
+  }
+  const int g_t = tid < NG * CT ? tid / NG : SCAN_CHUNK_MAX;
+  const int g_g = g_t * NG * H + (tid - g_t * NG) * H + head;
   auto fetch = [&](int t0) {                         // chunk starting at token t0 -> registers
     const int n = min(CT, last - t0);
+    const size_t row0 = (size_t)t0 * p.ld;
 #pragma unroll
     for (int j = 0; j < SCAN_KQ_REGS; ++j) {
-      const int idx = tid + j * nthreads;
-      const int t = idx / dk, e = idx - t * dk;
       fk[j] = fq[j] = 0.f;
-      if (t < n) {
-        const size_t row = (size_t)(t0 + t) * p.ld;
-        fk[j] = to_f32(kg[row + e]);
-        fq[j] = to_f32(qg[row + e]) * p.q_scale;
+      if (kq_t[j] < n) {
+        fk[j] = to_f32(kg[row0 + kq_g[j]]);
+        fq[j] = to_f32(qg[row0 + kq_g[j]]) * p.q_scale;
       }
     }
 #pragma unroll
-    for (int j = 0; j < SCAN_V_REGS; ++j) {
-      const int idx = tid + j * nthreads;
-      const int t = idx / cols, cc = idx - t * cols;
-      fv[j] = (t < n && cc < v_left) ? to_f32(vg[(size_t)(t0 + t) * p.ld + cc]) : 0.f;
-    }
-    if (tid < 2 * CT) {
-      const int t = tid >> 1;
-      fg = t < n ? p.gates[(size_t)(t0 + t) * 2 * H + (tid & 1) * H + head] : 0.f;
-    }
+    for (int j = 0; j < SCAN_V_REGS; ++j) fv[j] = v_t[j] < n ? to_f32(vg[row0 + v_g[j]]) : 0.f;
+    fg = g_t < n ? p.gates[(size_t)t0 * NG * H + g_g] : 0.f;
   };
   auto stage = [&](float* buf) {                     // registers -> LDS
 #pragma unroll
     for (int j = 0; j < SCAN_KQ_REGS; ++j) {
-      const int idx = tid + j * nthreads;
-      const int t = idx / dk, e = idx - t * dk;
-      if (t < CT) {
-        float* row = buf + (size_t)t * 2 * R * PITCH + (e / NPL) * PITCH + (e % NPL);
-        row[0] = fk[j];
-        row[R * PITCH] = fq[j];
+      if (kq_t[j] < SCAN_CHUNK_MAX) {
+        buf[kq_l[j]] = fk[j];
+        buf[kq_l[j] + R * PITCH] = fq[j];
       }
     }
 #pragma unroll
@@ -150,19 +172,17 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
       const int idx = tid + j * nthreads;
       if (idx < v_floats) buf[kq_floats + idx] = fv[j];
     }
-    if (tid < 2 * CT) buf[kq_floats + v_floats + tid] = fg;
+    if (tid < NG * CT) buf[kq_floats + v_floats + tid] = fg;
   };
   float* st = p.state + (size_t)slot * p.slot_stride + (size_t)(head * p.waves_per_head + (active ? w : 0)) * p.wave_floats;
   const bool zero = p.fresh[seq] != 0;
   float S[NPL], nrm[NPL];
-  float m = 0.f;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     S[i] = (zero || !active) ? 0.f : st[i * RA_WAVE + lane];
     nrm[i] = 0.f;
     if (MEMORY && !zero && active) nrm[i] = st[NPL * RA_WAVE + i * R + r];
   }
-  if (MEMORY && !zero && active) m = st[NPL * RA_WAVE + NPL * R];
   fetch(first);
   __syncthreads();                                   // the zero fill is done
   stage(lds);
@@ -174,48 +194,55 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     const float* buf = lds + (size_t)which * buf_floats;
     const int n = min(CT, last - t0);
     if (active) {
-#pragma unroll 2
-      for (int tt = 0; tt < n; ++tt) {
+      const int vcol = (tid / RA_WAVE) * CPW + c;
+      float nk[NPL], nq[NPL], nv, ng0, ng1, ng2 = 0.f;
+      auto read = [&](int tt) {                      // a token's operands out of LDS
         const float* kp = buf + (size_t)tt * 2 * R * PITCH + r * PITCH;
         const float* qp = kp + R * PITCH;
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) { nk[i] = kp[i]; nq[i] = qp[i]; }
+        nv = buf[kq_floats + tt * cols + vcol];
+        ng0 = buf[kq_floats + v_floats + NG * tt];
+        ng1 = buf[kq_floats + v_floats + NG * tt + 1];
+        if (MEMORY) ng2 = buf[kq_floats + v_floats + NG * tt + 2];
+      };
+      read(0);
+      for (int tt = 0; tt < n; ++tt) {
         float k[NPL], q[NPL];
 #pragma unroll
-        for (int i = 0; i < NPL; ++i) { k[i] = kp[i]; q[i] = qp[i]; }
-        const float v = buf[kq_floats + tt * cols + (tid / RA_WAVE) * CPW + c];
-        const float g0 = buf[kq_floats + v_floats + 2 * tt], g1 = buf[kq_floats + v_floats + 2 * tt + 1];
+        for (int i = 0; i < NPL; ++i) { k[i] = nk[i]; q[i] = nq[i]; }
+        const float v = nv, g0 = ng0, g1 = ng1, g2 = ng2;
+        if (tt + 1 < n) read(tt + 1);                // asked for before this token's arithmetic
         float o;
         if (MEMORY) {
-          const float m_new = fmaxf(g1 + m, g0);
-          const float keep = expf(g1 + m - m_new);
-          const float take = expf(g0 - m_new);
-          m = m_new;
-          float ps = 0.f, pn = 0.f;
+          const float keep = g0, take = g1;
+          float ps[2] = {0.f, 0.f}, pn[2] = {0.f, 0.f};
 #pragma unroll
           for (int i = 0; i < NPL; ++i) {
             const float tk = take * k[i];
             nrm[i] = keep * nrm[i] + tk;
             S[i] = keep * S[i] + tk * v;
-            ps += S[i] * q[i];
-            pn += nrm[i] * q[i];
+            ps[i & 1] += S[i] * q[i];
+            pn[i & 1] += nrm[i] * q[i];
           }
-          ps = group_sum<R>(ps);
-          pn = group_sum<R>(pn);
-          o = ps / (fmaxf(fabsf(pn), expf(-m)) + p.denom_eps);
+          const float s1 = group_sum<R>(ps[0] + ps[1]);
+          const float s2 = group_sum<R>(pn[0] + pn[1]);
+          o = s1 / (fmaxf(fabsf(s2), g2) + p.denom_eps);
         } else {
-          float pa = 0.f, pb = 0.f, pkq = 0.f;
+          float pa[2] = {0.f, 0.f}, pb[2] = {0.f, 0.f}, pkq[2] = {0.f, 0.f};
 #pragma unroll
           for (int i = 0; i < NPL; ++i) {
-            pa += S[i] * k[i];
-            pb += S[i] * q[i];
-            pkq += k[i] * q[i];
+            pa[i & 1] += S[i] * k[i];
+            pb[i & 1] += S[i] * q[i];
+            pkq[i & 1] += k[i] * q[i];
           }
-          pa = group_sum<R>(pa);
-          pb = group_sum<R>(pb);
-          pkq = group_sum<R>(pkq);
-          const float u = g0 * (v - g1 * pa);
+          const float sa = group_sum<R>(pa[0] + pa[1]);
+          const float sb = group_sum<R>(pb[0] + pb[1]);
+          const float skq = group_sum<R>(pkq[0] + pkq[1]);
+          const float u = g0 * (v - g1 * sa);
 #pragma unroll
           for (int i = 0; i < NPL; ++i) S[i] = g1 * S[i] + k[i] * u;
-          o = g1 * pb + u * pkq;
+          o = g1 * sb + u * skq;
         }
         if (col_ok && r == 0) p.out[(size_t)(t0 + tt) * ow + head * dv + col] = o;
       }
@@ -230,18 +257,67 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     st[i * RA_WAVE + lane] = S[i];
     if (MEMORY && c == 0) st[NPL * RA_WAVE + i * R + r] = nrm[i];
   }
-  if (MEMORY && lane == 0) st[NPL * RA_WAVE + NPL * R] = m;
 }
 
-// lg[t, h] <- cap tanh((z + bias) / cap);  lg[t, H + h] <- log sigmoid(cap tanh((z + bias) / cap)), in place
-__global__ void matrix_memory_gates_kernel(float* __restrict__ lg, const float* __restrict__ bias, int H, float cap,
-                                           long n) {
-  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const int j = (int)(i % (2 * H));
-  float z = lg[i] + bias[j];
-  if (cap > 0.f) z = cap * tanhf(z / cap);
-  lg[i] = j < H ? z : logsigmoid_f(z);
+// The matrix memory's gates. z [T, 2 H] holds the pre-activations (input | forget); with a = cap tanh((z_i + bias) / cap)
+// and b = log sigmoid(cap tanh((z_f + bias) / cap)) the running maximum is m_t = max(b_t + m_{t-1}, a_t), a chain over
+// the request's tokens. The map m -> max(b + m, a) is the pair (a, b), and two such maps compose to
+// (max(a1 + b2, a2), b1 + b2), so a workgroup a (request, head) takes 256 tokens at a time through a prefix scan
+// in LDS. g3 [T, 3 H] gets keep = exp(b + m_{t-1} - m_t), take = exp(a - m_t) and exp(-m_t). The maximum itself
+// is kept in the request's state at `m_off` floats behind the head's first float (0 at a request's start).
+__global__ __launch_bounds__(256) void matrix_memory_gate_scan_kernel(
+    const float* __restrict__ z, const float* __restrict__ bias, float cap, float* __restrict__ g3,
+    float* __restrict__ state, long slot_stride, long head_floats, long m_off, const int* __restrict__ cu_tokens,
+    const int* __restrict__ state_slots, const int* __restrict__ fresh, int H) {
+  __shared__ float sA[256], sB[256];
+  const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+  const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+  const int slot = state_slots[seq];
+  if (slot < 0 || first >= last) return;       // the scan writes zeros for a padding row without reading its gates
+  float* mp = state + (size_t)slot * slot_stride + (size_t)head * head_floats + m_off;
+  float m_run = fresh[seq] != 0 ? 0.f : *mp;
+  for (int t0 = first; t0 < last; t0 += 256) {
+    const int t = t0 + tid;
+    const bool valid = t < last;
+    float a = -INFINITY, b = 0.f;              // the identity map for rows past the end
+    if (valid) {
+      float zi = z[(size_t)t * 2 * H + head] + bias[head];
+      float zf = z[(size_t)t * 2 * H + H + head] + bias[H + head];
+      if (cap > 0.f) { zi = cap * tanhf(zi / cap); zf = cap * tanhf(zf / cap); }
+      a = zi;
+      b = logsigmoid_f(zf);
+    }
+    float A = a, B = b;
+    sA[tid] = A;
+    sB[tid] = B;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+      float A1 = -INFINITY, B1 = 0.f;
+      const bool has = tid >= off;
+      if (has) { A1 = sA[tid - off]; B1 = sB[tid - off]; }
+      __syncthreads();
+      if (has) {                               // the earlier map first, then this one
+        A = fmaxf(A1 + B, A);
+        B = B1 + B;
+        sA[tid] = A;
+        sB[tid] = B;
+      }
+      __syncthreads();
+    }
+    const float m_t = fmaxf(B + m_run, A);
+    const float m_prev = tid == 0 ? m_run : fmaxf(sB[tid - 1] + m_run, sA[tid - 1]);
+    if (valid) {
+      float* o = g3 + (size_t)t * 3 * H + head;
+      o[0] = expf(b + m_prev - m_t);
+      o[H] = expf(a - m_t);
+      o[2 * H] = expf(-m_t);
+    }
+    const int end = min(255, last - 1 - t0);
+    const float m_end = fmaxf(sB[end] + m_run, sA[end]);
+    __syncthreads();                           // before the next round overwrites the maps
+    m_run = m_end;
+  }
+  if (tid == 0) *mp = m_run;
 }
 
 // gb[t, h] <- sigmoid(b);  gb[t, H + h] <- exp(-exp(A_log[h]) softplus(a + dt_bias[h])), in place
@@ -450,7 +526,7 @@ ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int dk) {
   if (ct > SCAN_KQ_REGS * L.threads / dk) ct = SCAN_KQ_REGS * L.threads / dk;
   if (ct > SCAN_V_REGS * L.threads / cols) ct = SCAN_V_REGS * L.threads / cols;
   if (ct > SCAN_LDS_FLOATS / per_token) ct = SCAN_LDS_FLOATS / per_token;
-  if (ct > L.threads / 2) ct = L.threads / 2;
+  if (ct > L.threads / 3) ct = L.threads / 3;
   if (ct < 1) ct = 1;
   L.chunk = ct;
   L.lds = (size_t)2 * ((size_t)ct * per_token) * sizeof(float);
@@ -464,10 +540,12 @@ int scan_dispatch(const ScanGeom& g, const ScanLaunch& L, const ScanArgs& a, hip
   do {                                             \
     if (g.NPL == 2) RA_SCAN(R, 2);                 \
     else if (g.NPL == 4) RA_SCAN(R, 4);            \
-    else if (g.NPL == 8) RA_SCAN(R, 8);            \
-    else RA_SCAN(R, 16);                           \
+    else RA_SCAN(R, 8);                            \
   } while (0)
-  if (g.R == 8) RA_SCAN_N(8); else RA_SCAN_N(32);
+  if (g.R == 8) RA_SCAN_N(8);
+  else if (g.R == 16) RA_SCAN_N(16);
+  else if (g.R == 32) RA_SCAN_N(32);
+  else RA_SCAN_N(64);
 #undef RA_SCAN_N
 #undef RA_SCAN
   return 0;
@@ -475,7 +553,8 @@ int scan_dispatch(const ScanGeom& g, const ScanLaunch& L, const ScanArgs& a, hip
 }  // namespace
 
 extern "C" int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, int q_off, int k_off, int v_off,
-                                     float* gates, const float* gate_bias, float* state, long slot_stride,
+                                     const float* gates, float* gates3, const float* gate_bias, float* state,
+                                     long slot_stride,
                                      const int* cu_tokens, const int* state_slots, const int* fresh, int n_seqs,
                                      int n_tokens, int heads, int key_dim, int value_dim, float gate_cap,
                                      float q_scale, float denom_eps, float* out, hipStream_t stream) {
@@ -488,8 +567,10 @@ extern "C" int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, in
            slot_stride, (long)heads * g.waves * g.wave_floats);
   RA_CHECK(heads <= 65535, "matrix_memory_scan: %d heads in one launch", heads);
   RA_CHECK(act_dtype == RA_F32 || act_dtype == RA_BF16, "matrix_memory_scan: unknown dtype tag %d", act_dtype);
-  const long n = (long)n_tokens * 2 * heads;
-  matrix_memory_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(gates, gate_bias, heads, gate_cap, n);
+  // the running maximum lives where the first wave of each head has its spare floats
+  matrix_memory_gate_scan_kernel<<<dim3(n_seqs, heads), 256, 0, stream>>>(
+      gates, gate_bias, gate_cap, gates3, state, slot_stride, (long)g.waves * g.wave_floats,
+      (long)g.NPL * RA_WAVE + (long)g.NPL * g.R, cu_tokens, state_slots, fresh, heads);
   RA_LAUNCH_CHECK("matrix_memory_gates");
   const ScanLaunch L = scan_launch(g, n_seqs, heads, key_dim);
   const size_t es = act_dtype == RA_F32 ? 4 : 2;
@@ -497,7 +578,7 @@ extern "C" int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, in
   a.q = (const char*)proj + (size_t)q_off * es;
   a.k = (const char*)proj + (size_t)k_off * es;
   a.v = (const char*)proj + (size_t)v_off * es;
-  a.ld = ld; a.q_heads = heads; a.gates = gates; a.state = state; a.slot_stride = slot_stride;
+  a.ld = ld; a.q_heads = heads; a.gates = gates3; a.state = state; a.slot_stride = slot_stride;
   a.cu_tokens = cu_tokens; a.state_slots = state_slots; a.fresh = fresh;
   a.H = heads; a.dk = key_dim; a.dv = value_dim; a.waves_per_head = g.waves; a.wave_floats = g.wave_floats;
   a.chunk = L.chunk; a.q_scale = q_scale; a.denom_eps = denom_eps; a.out = out;

@@ -230,10 +230,11 @@ int ra_gemm_wide_scaled(const void* A, const void* W, float* C, int M, int N, in
 // ---- recurrent mixers (recurrent.hip) ----
 // floats of state a request slot holds for the scan kernels; kind 0: matrix memory, 1: delta rule; -1: sizes not taken
 long ra_scan_state_floats(int kind, int heads, int key_dim, int value_dim);
-// gates [n_tokens, 2 heads] float pre-activations (input | forget), turned into log gates in place; proj rows hold
-// q, k (heads x key_dim) and v (heads x value_dim) at the given column offsets; out float [n_tokens, heads * value_dim]
-int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, int q_off, int k_off, int v_off, float* gates,
-                          const float* gate_bias, float* state, long slot_stride, const int* cu_tokens,
+// gates [n_tokens, 2 heads] float pre-activations (input | forget); gates3 [n_tokens, 3 heads] scratch for the
+// decay, input and threshold factors made from them; proj rows hold q, k (heads x key_dim) and v (heads x value_dim)
+// at the given column offsets; out float [n_tokens, heads * value_dim]
+int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, int q_off, int k_off, int v_off, const float* gates,
+                          float* gates3, const float* gate_bias, float* state, long slot_stride, const int* cu_tokens,
                           const int* state_slots, const int* fresh, int n_seqs, int n_tokens, int heads, int key_dim,
                           int value_dim, float gate_cap, float q_scale, float denom_eps, float* out,
                           hipStream_t stream);

@@ -1014,9 +1014,8 @@ class HipKernels:
                            out: torch.Tensor) -> None:
         """The matrix memory over the step's tokens, request by request in order, from and into ``state``
         [slots, floats]. ``proj`` [T, *] holds q and k (heads x key_dim) and v (heads x value_dim) from the
-        given columns; ``gates`` float32 [T, 2 heads] holds the input and forget gates' pre-activations and
-        is overwritten with the log gates; ``out`` float32 [T, heads * value_dim] gets the read-out before
-        its norm."""
+        given columns; ``gates`` float32 [T, 2 heads] holds the input and forget gates' pre-activations;
+        ``out`` float32 [T, heads * value_dim] gets the read-out before its norm."""
         _dev(proj, gates, gate_bias, state, out)
         T = proj.shape[0]
         self._check_scan("matrix_memory_scan", state, batch, T)
@@ -1028,8 +1027,10 @@ class HipKernels:
             raise ValueError("matrix_memory_scan: gates float32 [T, 2 heads], their bias float32 [2 heads]")
         if out.shape != (T, heads * value_dim) or out.dtype != torch.float32 or not out.is_contiguous():
             raise ValueError("matrix_memory_scan: out is contiguous float32 [T, heads * value_dim]")
+        factors = torch.empty((T, 3 * heads), dtype=torch.float32, device=proj.device)     # decay, input, threshold
         library.call("ra_matrix_memory_scan", proj.data_ptr(), _tag(proj, "matrix_memory_scan"), proj.stride(0),
-                     int(q_off), int(k_off), int(v_off), gates.data_ptr(), gate_bias.data_ptr(), state.data_ptr(),
+                     int(q_off), int(k_off), int(v_off), gates.data_ptr(), factors.data_ptr(), gate_bias.data_ptr(),
+                     state.data_ptr(),
                      state.stride(0), batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), batch.fresh.data_ptr(),
                      batch.num_seqs, T, int(heads), int(key_dim), int(value_dim), float(gate_cap), float(q_scale),
                      float(denom_eps), out.data_ptr(), _stream())
