@@ -116,7 +116,6 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
   // LDS: two buffers of [CT][2][R][PITCH] k and q, [CT][cols] v, [CT][NG] gates
   const int kq_floats = CT * 2 * R * PITCH, v_floats = CT * cols;
   const int buf_floats = kq_floats + v_floats + CT * NG;
-  for (int i = tid; i < 2 * buf_floats; i += nthreads) lds[i] = 0.f;      // the padding stays zero
   const int qh = head / (H / p.q_heads);
   const TA* qg = (const TA*)p.q + (size_t)qh * dk;
   const TA* kg = (const TA*)p.k + (size_t)qh * dk;
@@ -126,11 +125,13 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
   // what this thread fetches for a chunk is the same for every chunk: token (of the chunk), offset behind the
   // chunk's first row, and place in LDS are worked out once
   int kq_t[SCAN_KQ_REGS], kq_g[SCAN_KQ_REGS], kq_l[SCAN_KQ_REGS];
+  bool kq_e[SCAN_KQ_REGS];
 #pragma unroll
   for (int j = 0; j < SCAN_KQ_REGS; ++j) {
     const int idx = tid + j * nthreads;
-    const int t = idx / dk, e = idx - t * dk;
+    const int t = idx / (R * NPL), e = idx - t * (R * NPL);      // e runs over the lanes' runs: past dk they hold zeros
     kq_t[j] = t < CT ? t : SCAN_CHUNK_MAX;           // past the chunk: never fetched, never stored
+    kq_e[j] = e < dk;
     kq_g[j] = t * p.ld + e;
     kq_l[j] = t * 2 * R * PITCH + (e / NPL) * PITCH + (e % NPL);
   }
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
 #pragma unroll
     for (int j = 0; j < SCAN_KQ_REGS; ++j) {
       fk[j] = fq[j] = 0.f;
-      if (kq_t[j] < n) {
+      if (kq_t[j] < n && kq_e[j]) {
         fk[j] = to_f32(kg[row0 + kq_g[j]]);
         fq[j] = to_f32(qg[row0 + kq_g[j]]) * p.q_scale;
       }
@@ -184,7 +185,6 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     if (MEMORY && !zero && active) nrm[i] = st[NPL * RA_WAVE + i * R + r];
   }
   fetch(first);
-  __syncthreads();                                   // the zero fill is done
   stage(lds);
   __syncthreads();
   int which = 0;
@@ -515,7 +515,7 @@ struct ScanLaunch {
   int threads, chunk;
   size_t lds;
 };
-ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int dk) {
+ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int max_q_len) {
   const int wpb = g.waves < 4 ? g.waves : 4;           // waves a workgroup
   ScanLaunch L;
   L.threads = wpb * RA_WAVE;
@@ -523,7 +523,8 @@ ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int dk) {
   const int cols = wpb * g.CPW;
   const int per_token = 2 * g.R * (g.NPL + 4) + cols + 2;
   int ct = SCAN_CHUNK_MAX;
-  if (ct > SCAN_KQ_REGS * L.threads / dk) ct = SCAN_KQ_REGS * L.threads / dk;
+  if (ct > SCAN_KQ_REGS * L.threads / (g.R * g.NPL)) ct = SCAN_KQ_REGS * L.threads / (g.R * g.NPL);
+  if (max_q_len > 0 && ct > max_q_len) ct = max_q_len;      // a step of single tokens stages one token
   if (ct > SCAN_V_REGS * L.threads / cols) ct = SCAN_V_REGS * L.threads / cols;
   if (ct > SCAN_LDS_FLOATS / per_token) ct = SCAN_LDS_FLOATS / per_token;
   if (ct > L.threads / 3) ct = L.threads / 3;
@@ -556,8 +557,8 @@ extern "C" int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, in
                                      const float* gates, float* gates3, const float* gate_bias, float* state,
                                      long slot_stride,
                                      const int* cu_tokens, const int* state_slots, const int* fresh, int n_seqs,
-                                     int n_tokens, int heads, int key_dim, int value_dim, float gate_cap,
-                                     float q_scale, float denom_eps, float* out, hipStream_t stream) {
+                                     int n_tokens, int max_q_len, int heads, int key_dim, int value_dim,
+                                     float gate_cap, float q_scale, float denom_eps, float* out, hipStream_t stream) {
   RA_CHECK(n_seqs > 0 && n_tokens > 0 && heads > 0, "matrix_memory_scan: %d requests, %d tokens, %d heads", n_seqs,
            n_tokens, heads);
   ScanGeom g;
@@ -572,7 +573,7 @@ extern "C" int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, in
       gates, gate_bias, gate_cap, gates3, state, slot_stride, (long)g.waves * g.wave_floats,
       (long)g.NPL * RA_WAVE + (long)g.NPL * g.R, cu_tokens, state_slots, fresh, heads);
   RA_LAUNCH_CHECK("matrix_memory_gates");
-  const ScanLaunch L = scan_launch(g, n_seqs, heads, key_dim);
+  const ScanLaunch L = scan_launch(g, n_seqs, heads, max_q_len);
   const size_t es = act_dtype == RA_F32 ? 4 : 2;
   ScanArgs a = {};
   a.q = (const char*)proj + (size_t)q_off * es;
@@ -623,8 +624,8 @@ extern "C" int ra_delta_rule_prepare(const void* proj, int act_dtype, int ld, co
 
 extern "C" int ra_delta_rule_scan(const float* qkv, int ld, float* gates, const float* a_log, const float* dt_bias,
                                   float* state, long slot_stride, const int* cu_tokens, const int* state_slots,
-                                  const int* fresh, int n_seqs, int n_tokens, int heads, int key_heads, int key_dim,
-                                  int value_dim, float* out, hipStream_t stream) {
+                                  const int* fresh, int n_seqs, int n_tokens, int max_q_len, int heads, int key_heads,
+                                  int key_dim, int value_dim, float* out, hipStream_t stream) {
   RA_CHECK(n_seqs > 0 && n_tokens > 0 && heads > 0 && key_heads > 0 && heads % key_heads == 0,
            "delta_rule_scan: %d requests, %d tokens, %d heads on %d key heads", n_seqs, n_tokens, heads, key_heads);
   ScanGeom g;
@@ -635,7 +636,7 @@ extern "C" int ra_delta_rule_scan(const float* qkv, int ld, float* gates, const 
   const long n = (long)n_tokens * 2 * heads;
   delta_rule_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(gates, a_log, dt_bias, heads, n);
   RA_LAUNCH_CHECK("delta_rule_gates");
-  const ScanLaunch L = scan_launch(g, n_seqs, heads, key_dim);
+  const ScanLaunch L = scan_launch(g, n_seqs, heads, max_q_len);
   ScanArgs a = {};
   a.q = qkv;
   a.k = qkv + (size_t)key_heads * key_dim;

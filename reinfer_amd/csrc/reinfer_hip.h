@@ -230,13 +230,14 @@ int ra_gemm_wide_scaled(const void* A, const void* W, float* C, int M, int N, in
 // ---- recurrent mixers (recurrent.hip) ----
 // floats of state a request slot holds for the scan kernels; kind 0: matrix memory, 1: delta rule; -1: sizes not taken
 long ra_scan_state_floats(int kind, int heads, int key_dim, int value_dim);
+// max_q_len: the most tokens a request brings (0: unknown; it only sizes the chunks that are staged)
 // gates [n_tokens, 2 heads] float pre-activations (input | forget); gates3 [n_tokens, 3 heads] scratch for the
 // decay, input and threshold factors made from them; proj rows hold q, k (heads x key_dim) and v (heads x value_dim)
 // at the given column offsets; out float [n_tokens, heads * value_dim]
 int ra_matrix_memory_scan(const void* proj, int act_dtype, int ld, int q_off, int k_off, int v_off, const float* gates,
                           float* gates3, const float* gate_bias, float* state, long slot_stride, const int* cu_tokens,
-                          const int* state_slots, const int* fresh, int n_seqs, int n_tokens, int heads, int key_dim,
-                          int value_dim, float gate_cap, float q_scale, float denom_eps, float* out,
+                          const int* state_slots, const int* fresh, int n_seqs, int n_tokens, int max_q_len, int heads,
+                          int key_dim, int value_dim, float gate_cap, float q_scale, float denom_eps, float* out,
                           hipStream_t stream);
 // proj rows hold q | k (key_heads x key_dim each) | v (heads x value_dim) from column 0; filt float [channels, taps];
 // the filter's tail lies at tail_off floats in a request's state slot; qkv float [n_tokens, channels]
@@ -247,7 +248,7 @@ int ra_delta_rule_prepare(const void* proj, int act_dtype, int ld, const float* 
 // gates [n_tokens, 2 heads] float pre-activations (b | a), turned into (beta | decay) in place
 int ra_delta_rule_scan(const float* qkv, int ld, float* gates, const float* a_log, const float* dt_bias, float* state,
                        long slot_stride, const int* cu_tokens, const int* state_slots, const int* fresh, int n_seqs,
-                       int n_tokens, int heads, int key_heads, int key_dim, int value_dim, float* out,
+                       int n_tokens, int max_q_len, int heads, int key_heads, int key_dim, int value_dim, float* out,
                        hipStream_t stream);
 int ra_head_norm_gate(const float* read, const float* weight, int per_head_weight, const void* gate, int ldg,
                       int act_dtype, int silu, float eps, int n_tokens, int heads, int value_dim, void* out,

@@ -60,9 +60,9 @@ _SIGNATURES = {
     "ra_moe_down_chosen": [P, P, P, P, P, I, I, I, I, I, I, P],
     "ra_moe_route_sigmoid": [P, I, I, I, I, I, I, F, P, P, I, P],
     "ra_moe_silu_gate_scale": [P, P, I, P, P, I, I, I, I, I, P],
-    "ra_matrix_memory_scan": [P, I, I, I, I, I, P, P, P, P, c_long, P, P, P, I, I, I, I, I, F, F, F, P, P],
+    "ra_matrix_memory_scan": [P, I, I, I, I, I, P, P, P, P, c_long, P, P, P, I, I, I, I, I, I, F, F, F, P, P],
     "ra_delta_rule_prepare": [P, I, I, P, P, c_long, c_long, P, P, P, P, I, I, I, I, I, I, I, F, F, P, P],
-    "ra_delta_rule_scan": [P, I, P, P, P, P, c_long, P, P, P, I, I, I, I, I, I, P, P],
+    "ra_delta_rule_scan": [P, I, P, P, P, P, c_long, P, P, P, I, I, I, I, I, I, I, P, P],
     "ra_head_norm_gate": [P, P, I, P, I, I, I, F, I, I, I, P, P],
     "ra_normed_mean": [P, P, I, I, F, I, I, P, P, F, P],
     "ra_stream_read": [P, c_long, P, P],

@@ -1032,8 +1032,8 @@ class HipKernels:
                      int(q_off), int(k_off), int(v_off), gates.data_ptr(), factors.data_ptr(), gate_bias.data_ptr(),
                      state.data_ptr(),
                      state.stride(0), batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), batch.fresh.data_ptr(),
-                     batch.num_seqs, T, int(heads), int(key_dim), int(value_dim), float(gate_cap), float(q_scale),
-                     float(denom_eps), out.data_ptr(), _stream())
+                     batch.num_seqs, T, int(getattr(batch, "max_q_len", 0) or 0), int(heads), int(key_dim),
+                     int(value_dim), float(gate_cap), float(q_scale), float(denom_eps), out.data_ptr(), _stream())
 
     def delta_rule_prepare(self, proj: torch.Tensor, filt: torch.Tensor, state: torch.Tensor, tail_off: int, batch,
                            key_heads: int, key_dim: int, heads: int, value_dim: int, taps: int, unit_eps: float,
@@ -1081,8 +1081,9 @@ class HipKernels:
             raise ValueError("delta_rule_scan: out is contiguous float32 [T, heads * value_dim]")
         library.call("ra_delta_rule_scan", qkv.data_ptr(), qkv.stride(0), gates.data_ptr(), a_log.data_ptr(),
                      dt_bias.data_ptr(), state.data_ptr(), state.stride(0), batch.cu_tokens.data_ptr(),
-                     batch.state_slots.data_ptr(), batch.fresh.data_ptr(), batch.num_seqs, T, int(heads),
-                     int(key_heads), int(key_dim), int(value_dim), out.data_ptr(), _stream())
+                     batch.state_slots.data_ptr(), batch.fresh.data_ptr(), batch.num_seqs, T,
+                     int(getattr(batch, "max_q_len", 0) or 0), int(heads), int(key_heads), int(key_dim), int(value_dim),
+                     out.data_ptr(), _stream())
 
     def head_norm_gate(self, read: torch.Tensor, weight: torch.Tensor, per_head: bool, gate: torch.Tensor, kind: str,
                        eps: float, heads: int, value_dim: int, out: torch.Tensor) -> None:
