@@ -122,9 +122,9 @@ class KobolixConfig:
     @staticmethod
     def _read_memory(m: Mapping[str, Any], where: str) -> KobolixMemoryMixer:
         at = _At(m, where)
-        cap = at.float("gate_cap")
-        if cap <= 0.0:
-            raise ConfigError(where + "gate_cap", "must be > 0")
+        cap = at.float("gate_cap", 0.0)                  # absent: the gates are not capped
+        if cap < 0.0:
+            raise ConfigError(where + "gate_cap", "must be > 0 (absent: no cap)")
         return KobolixMemoryMixer(heads=at.int("heads", minimum=1), dim=at.int("dim", minimum=1),
                                   vdim=at.int("vdim", minimum=1), gate_cap=cap)
 
@@ -145,7 +145,7 @@ class KobolixConfig:
             if dims % 2 or dims > dim:
                 raise ConfigError(where + "rot.dims", f"{dims} entries in pairs out of {dim}")
         return KobolixAttention(heads=heads, kv_heads=kv, dim=dim, vdim=at.int("vdim", minimum=1),
-                                scale=at.float("scale"), rot_base=base, rot_dims=dims)
+                                scale=at.float("scale", float(dim) ** -0.5), rot_base=base, rot_dims=dims)
 
     @staticmethod
     def _read_delta(m: Mapping[str, Any], where: str) -> KobolixDeltaRule:
@@ -208,11 +208,16 @@ class KobolixConfig:
         for L in self.layers:
             if L.kind == "mlstm":
                 m = L.mixer
-                mixer: Dict[str, Any] = {"dim": m.dim, "gate_cap": m.gate_cap, "heads": m.heads, "vdim": m.vdim}
+                mixer: Dict[str, Any] = {"dim": m.dim, "heads": m.heads, "vdim": m.vdim}
+                if m.gate_cap:
+                    mixer["gate_cap"] = m.gate_cap
             else:
                 a, d = L.mixer.left, L.mixer.right
-                mixer = {"left": {"dim": a.dim, "heads": a.heads, "kv_heads": a.kv_heads,
-                                  "rot": {"base": a.rot_base, "dims": a.rot_dims}, "scale": a.scale, "vdim": a.vdim},
+                left: Dict[str, Any] = {"dim": a.dim, "heads": a.heads, "kv_heads": a.kv_heads, "scale": a.scale,
+                                        "vdim": a.vdim}
+                if a.rot_dims:
+                    left["rot"] = {"base": a.rot_base, "dims": a.rot_dims}
+                mixer = {"left": left,
                          "right": {"conv": d.conv, "dim": d.dim, "heads": d.heads, "kv_heads": d.kv_heads,
                                    "vdim": d.vdim}}
             mlp: Any = None

@@ -175,8 +175,9 @@ class KernelDouble:
                            denom_eps, out):
         p = proj.float()
         z = gates + gate_bias
-        a_in = cap * torch.tanh(z[:, :H] / cap)
-        b_f = torch.nn.functional.logsigmoid(cap * torch.tanh(z[:, H:] / cap))
+        if cap > 0:
+            z = cap * torch.tanh(z / cap)
+        a_in, b_f = z[:, :H], torch.nn.functional.logsigmoid(z[:, H:])
         nS = H * dk * dv
         for first, rows, slot, fresh in self._requests(batch):
             if slot < 0:

@@ -78,14 +78,25 @@ KB_C = {
     "architecture": "Kobolix", "vocab": 257, "width": 96, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
     "embedding": {"scale": 2.0},
     "layers": [
-        {"type": "mlstm", "mixer": _memory(2, 32, 48, 12.0), "mlp": _moe(4, 4, 32, scale=0.5, shared=16)},
+        {"type": "mlstm", "mixer": _memory(2, 32, 48, 11.0), "mlp": _moe(4, 4, 32, scale=0.5, shared=16)},
         {"type": "parallel", "mixer": {"left": _attn(8, 1, 32, 32, 8, base=100000.0), "right": _delta(6, 3, 16, 24, 4)},
          "mlp": _dense(128)},
         {"type": "parallel", "mixer": {"left": _attn(3, 3, 40, 24, 40), "right": _delta(1, 1, 64, 40, 2)},
          "mlp": None},
     ],
 }
-CONFIGS = {"A": (KB_A, 21), "B": (KB_B, 22), "C": (KB_C, 23)}
+# whatever may be absent is absent: no rotation, no cap on the gates, no score scale given (1 / sqrt(size)), no groups,
+# no router scale, no shared expert, no embedding scale, no residual factor; one expert of one; a side-by-side layer first
+KB_D = {
+    "architecture": "Kobolix", "vocab": 90, "width": 40, "norm": {"eps": 1e-6},
+    "layers": [
+        {"type": "parallel", "mixer": {"left": {"dim": 16, "heads": 5, "kv_heads": 5, "vdim": 8},
+                                       "right": _delta(3, 1, 8, 16, 2)},
+         "mlp": {"expert": {"ff": 24}, "kind": "moe", "router": {"experts": 1, "top": 1}}},
+        {"type": "mlstm", "mixer": {"dim": 8, "heads": 5, "vdim": 8}, "mlp": _dense(56)},
+    ],
+}
+CONFIGS = {"A": (KB_A, 21), "B": (KB_B, 22), "C": (KB_C, 23), "D": (KB_D, 24)}
 
 # deviation of the random matrices by the last part of their name
 STD = {"embed": 0.5, "router": 0.5, "conv": 0.6, "i": 0.3, "f": 0.3, "a": 0.3, "b": 0.3, "default": 0.15}

@@ -46,13 +46,14 @@ def logsigmoid(z):
 # ------------------------------------------------------------------ matrix memory (mLSTM)
 def mlstm(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, cfg: dict, eps: float) -> torch.Tensor:
     """h [T, width] -> [T, width]. State per head: S [dim, vdim], n [dim], m (scalar, starts at 0)."""
-    H, dk, dv, cap = cfg["heads"], cfg["dim"], cfg["vdim"], float(cfg["gate_cap"])
+    H, dk, dv, cap = cfg["heads"], cfg["dim"], cfg["vdim"], cfg.get("gate_cap")
     T = h.shape[0]
     q = (h @ w[p + "q"].T).view(T, H, dk) * dk ** -0.5
     k = (h @ w[p + "k"].T).view(T, H, dk)
     v = (h @ w[p + "v"].T).view(T, H, dv)
-    gi = cap * torch.tanh((h @ w[p + "i"].T + w[p + "i.b"]) / cap)                     # [T, H] log input gate
-    gf = logsigmoid(cap * torch.tanh((h @ w[p + "f"].T + w[p + "f.b"]) / cap))         # [T, H] log forget gate
+    soft = (lambda z: float(cap) * torch.tanh(z / float(cap))) if cap else (lambda z: z)      # no cap given: none
+    gi = soft(h @ w[p + "i"].T + w[p + "i.b"])                                         # [T, H] log input gate
+    gf = logsigmoid(soft(h @ w[p + "f"].T + w[p + "f.b"]))                             # [T, H] log forget gate
     out = torch.zeros(T, H, dv, dtype=D)
     for a in range(H):
         S = torch.zeros(dk, dv, dtype=D)
@@ -98,7 +99,7 @@ def attention(h, w, p, cfg) -> torch.Tensor:
     out = torch.zeros(T, H, dv, dtype=D)
     for a in range(H):
         g = a // (H // G)
-        s = (q[:, a] @ k[:, g].T) * cfg["scale"]
+        s = (q[:, a] @ k[:, g].T) * cfg.get("scale", dk ** -0.5)
         s = s.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float("-inf"))
         out[:, a] = torch.softmax(s, dim=-1) @ v[:, g]
     return out.reshape(T, H * dv) @ w[p + "o"].T

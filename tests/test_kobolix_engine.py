@@ -78,7 +78,8 @@ def test_configuration_errors_name_the_key():
             node[path[-1]] = value
         return raw
     for path, value, key in ((["width"], None, "width"), (["norm", "eps"], None, "norm.eps"),
-                             (["layers", 1, "mixer", "gate_cap"], None, "layers[1].mixer.gate_cap"),
+                             (["layers", 1, "mixer", "gate_cap"], -2.0, "layers[1].mixer.gate_cap"),
+                             (["layers", 1, "mixer", "vdim"], None, "layers[1].mixer.vdim"),
                              (["layers", 1, "type"], "conv", "layers[1].type"),
                              (["layers", 0, "mixer", "left", "kv_heads"], 3, "layers[0].mixer.left.kv_heads"),
                              (["layers", 0, "mixer", "left", "rot", "dims"], 26, "layers[0].mixer.left.rot.dims"),
@@ -191,7 +192,7 @@ CHECKS = [check_whole_and_one_by_one, check_portions, check_mixed_with_reuse, ch
 
 # ------------------------------------------------------------------ CPU: bookkeeping on the stand-in
 @pytest.mark.parametrize("check", CHECKS, ids=lambda f: f.__name__)
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_engine_bookkeeping_cpu(tmp_path_factory, check, which):
     folder = make_folder(tmp_path_factory.getbasetemp(), which, "float32")
     with kernels.use(KernelDouble()):
@@ -247,7 +248,8 @@ def test_sharp_attention_and_long_memory_cpu(tmp_path_factory):
 
 
 # ------------------------------------------------------------------ GPU: the real kernels
-GPU_CASES = [("A", "float32"), ("B", "float32"), ("C", "float32"), ("C", "bfloat16"), ("B", "bfloat16")]
+GPU_CASES = [("A", "float32"), ("B", "float32"), ("C", "float32"), ("D", "float32"), ("C", "bfloat16"), ("B", "bfloat16"),
+             ("D", "bfloat16")]
 
 
 @pytest.mark.gpu
