@@ -241,9 +241,10 @@ def test_trace_run_puresun(tmp_path, which, dtype):
 
 @pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "bfloat16"), ("B", "float32")])
 def test_trace_run_kobolix(tmp_path, which, dtype):
-    """A design with recurrent layers through the same program: five requests on four state slots and 192 tokens
-    of cache (none, for the configuration that keeps no keys), portions beside single tokens, a request left out
-    of a step, slots and blocks taken again."""
+    """A design with recurrent layers through the same program: five requests on four state slots and a cache for
+    the 320 tokens that the four live ones hold at most, each rounded up to 64 (no cache at all for the
+    configuration that keeps no keys), portions beside single tokens, a request left out of a step, slots and blocks
+    taken again."""
     import kobolix_helpers as kh
     import plain_kobolix
     from test_kobolix_engine import assert_close
@@ -269,7 +270,7 @@ def test_trace_run_kobolix(tmp_path, which, dtype):
     out = tmp_path / f"out_{dtype}"
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-         "--out", str(out), "--max-tokens", "192"],
+         "--out", str(out), "--max-tokens", "320"],
         input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(len(plan))]
