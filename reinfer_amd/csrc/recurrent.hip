@@ -195,56 +195,62 @@ __global__ __launch_bounds__(256) void scan_kernel(ScanArgs p) {
     const int n = min(CT, last - t0);
     if (active) {
       const int vcol = (tid / RA_WAVE) * CPW + c;
-      float nk[NPL], nq[NPL], nv, ng0, ng1, ng2 = 0.f;
-      auto read = [&](int tt) {                      // a token's operands out of LDS
+      struct Operands { float k[NPL], q[NPL], v, g0, g1, g2; };
+      auto read = [&](int tt, Operands& x) {         // a token's operands out of LDS
         const float* kp = buf + (size_t)tt * 2 * R * PITCH + r * PITCH;
         const float* qp = kp + R * PITCH;
 #pragma unroll
-        for (int i = 0; i < NPL; ++i) { nk[i] = kp[i]; nq[i] = qp[i]; }
-        nv = buf[kq_floats + tt * cols + vcol];
-        ng0 = buf[kq_floats + v_floats + NG * tt];
-        ng1 = buf[kq_floats + v_floats + NG * tt + 1];
-        if (MEMORY) ng2 = buf[kq_floats + v_floats + NG * tt + 2];
+        for (int i = 0; i < NPL; ++i) { x.k[i] = kp[i]; x.q[i] = qp[i]; }
+        x.v = buf[kq_floats + tt * cols + vcol];
+        x.g0 = buf[kq_floats + v_floats + NG * tt];
+        x.g1 = buf[kq_floats + v_floats + NG * tt + 1];
+        x.g2 = MEMORY ? buf[kq_floats + v_floats + NG * tt + 2] : 0.f;
       };
-      read(0);
-      for (int tt = 0; tt < n; ++tt) {
-        float k[NPL], q[NPL];
-#pragma unroll
-        for (int i = 0; i < NPL; ++i) { k[i] = nk[i]; q[i] = nq[i]; }
-        const float v = nv, g0 = ng0, g1 = ng1, g2 = ng2;
-        if (tt + 1 < n) read(tt + 1);                // asked for before this token's arithmetic
+      auto step = [&](int tt, const Operands& x) {   // one token: the state moves on, the read-out is stored
         float o;
         if (MEMORY) {
-          const float keep = g0, take = g1;
+          const float keep = x.g0, take = x.g1;
           float ps[2] = {0.f, 0.f}, pn[2] = {0.f, 0.f};
 #pragma unroll
           for (int i = 0; i < NPL; ++i) {
-            const float tk = take * k[i];
+            const float tk = take * x.k[i];
             nrm[i] = keep * nrm[i] + tk;
-            S[i] = keep * S[i] + tk * v;
-            ps[i & 1] += S[i] * q[i];
-            pn[i & 1] += nrm[i] * q[i];
+            S[i] = keep * S[i] + tk * x.v;
+            ps[i & 1] += S[i] * x.q[i];
+            pn[i & 1] += nrm[i] * x.q[i];
           }
           const float s1 = group_sum<R>(ps[0] + ps[1]);
           const float s2 = group_sum<R>(pn[0] + pn[1]);
-          o = s1 / (fmaxf(fabsf(s2), g2) + p.denom_eps);
+          o = __fdividef(s1, fmaxf(fabsf(s2), x.g2) + p.denom_eps);      // a reciprocal and a product: within an ulp or two
         } else {
           float pa[2] = {0.f, 0.f}, pb[2] = {0.f, 0.f}, pkq[2] = {0.f, 0.f};
 #pragma unroll
           for (int i = 0; i < NPL; ++i) {
-            pa[i & 1] += S[i] * k[i];
-            pb[i & 1] += S[i] * q[i];
-            pkq[i & 1] += k[i] * q[i];
+            pa[i & 1] += S[i] * x.k[i];
+            pb[i & 1] += S[i] * x.q[i];
+            pkq[i & 1] += x.k[i] * x.q[i];
           }
           const float sa = group_sum<R>(pa[0] + pa[1]);
           const float sb = group_sum<R>(pb[0] + pb[1]);
           const float skq = group_sum<R>(pkq[0] + pkq[1]);
-          const float u = g0 * (v - g1 * sa);
+          const float u = x.g0 * (x.v - x.g1 * sa);
 #pragma unroll
-          for (int i = 0; i < NPL; ++i) S[i] = g1 * S[i] + k[i] * u;
-          o = g1 * sb + u * skq;
+          for (int i = 0; i < NPL; ++i) S[i] = x.g1 * S[i] + x.k[i] * u;
+          o = x.g1 * sb + u * skq;
         }
         if (col_ok && r == 0) p.out[(size_t)(t0 + tt) * ow + head * dv + col] = o;
+      };
+      // two sets of operand registers take turns: a token's operands are asked for before the arithmetic of the
+      // token before it, and nothing is copied
+      Operands xa, xb;
+      read(0, xa);
+      for (int tt = 0; tt < n; tt += 2) {
+        if (tt + 1 < n) read(tt + 1, xb);
+        step(tt, xa);
+        if (tt + 1 < n) {
+          if (tt + 2 < n) read(tt + 2, xa);
+          step(tt + 1, xb);
+        }
       }
     }
     if (more) stage(lds + (size_t)(which ^ 1) * buf_floats);
