@@ -527,7 +527,7 @@ ScanLaunch scan_launch(const ScanGeom& g, int n_seqs, int heads, int max_q_len) 
   L.threads = wpb * RA_WAVE;
   L.grid = dim3(n_seqs, heads, (g.waves + wpb - 1) / wpb);
   const int cols = wpb * g.CPW;
-  const int per_token = 2 * g.R * (g.NPL + 4) + cols + 2;
+  const int per_token = 2 * g.R * (g.NPL + 4) + cols + 3;      // k and q runs, the columns of v, up to 3 gate numbers
   int ct = SCAN_CHUNK_MAX;
   if (ct > SCAN_KQ_REGS * L.threads / (g.R * g.NPL)) ct = SCAN_KQ_REGS * L.threads / (g.R * g.NPL);
   if (max_q_len > 0 && ct > max_q_len) ct = max_q_len;      // a step of single tokens stages one token

@@ -26,8 +26,9 @@ def make_batch(q_lens, slots, fresh, device):
                            fresh=i32(fresh), seq_of_token=i32(seq_of), q_lens=list(q_lens))
 
 
-# three calls: slots 2 and 0 start; they go on beside a padding row; slot 2 starts afresh beside slot 0 going on
-CALLS = [([5, 3], [2, 0], [1, 1]), ([1, 1, 4], [2, -1, 0], [0, 0, 0]), ([7, 2], [2, 0], [1, 0])]
+# four calls: slots 2 and 0 start; they go on beside a padding row; slot 2 starts afresh beside slot 0 going on; both go
+# on with portions of several staged chunks, the last of them part full
+CALLS = [([5, 3], [2, 0], [1, 1]), ([1, 1, 4], [2, -1, 0], [0, 0, 0]), ([7, 2], [2, 0], [1, 0]), ([53, 1, 40], [0, 3, 2], [0, 1, 0])]
 
 
 def close(got, ref, tol, what):
@@ -37,7 +38,7 @@ def close(got, ref, tol, what):
     assert err < tol, (what, err)
 
 
-@pytest.mark.parametrize("H,dk,dv", [(2, 40, 72), (3, 20, 28), (1, 136, 8), (2, 128, 40), (1, 8, 3), (2, 300, 17)])
+@pytest.mark.parametrize("H,dk,dv", [(2, 40, 72), (3, 20, 28), (1, 136, 8), (2, 128, 40), (1, 8, 3), (2, 300, 17), (5, 12, 70), (2, 4, 20)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_matrix_memory_scan(H, dk, dv, dtype):
     ops, ref = kernels.current(), KernelDouble()
@@ -63,7 +64,7 @@ def test_matrix_memory_scan(H, dk, dv, dtype):
         assert torch.equal(torch.nan_to_num(st_gpu[untouched], nan=7.0), torch.nan_to_num(before[untouched], nan=7.0))
 
 
-@pytest.mark.parametrize("H,G,dk,dv,taps", [(4, 2, 32, 48, 4), (4, 1, 20, 12, 3), (2, 2, 136, 8, 1), (1, 1, 16, 70, 2),
+@pytest.mark.parametrize("H,G,dk,dv,taps", [(4, 2, 32, 48, 4), (4, 1, 20, 12, 3), (2, 2, 136, 8, 1), (1, 1, 16, 70, 2), (4, 2, 16, 50, 4),
                                             (6, 3, 130, 9, 5)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_delta_rule_prepare_and_scan(H, G, dk, dv, taps, dtype):
